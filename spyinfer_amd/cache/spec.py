@@ -57,6 +57,14 @@ class PagedKVLayer:
         self.num_pages = k.shape[0]
 
 
+class PagedRowsLayer:
+    """One layer's part of a group of rows per token: ``rows [pages, page, width]``."""
+
+    def __init__(self, group: int, rows: torch.Tensor, page_size: int):
+        self.group, self.rows, self.page_size = group, rows, page_size
+        self.num_pages = rows.shape[0]
+
+
 class StateLayer:
     def __init__(self, group: int, state: torch.Tensor):
         self.group = group
@@ -91,9 +99,30 @@ class PagedKV(CacheKind):
 
 
 @dataclasses.dataclass(frozen=True)
+class PagedRows(CacheKind):
+    """One row of ``width`` values per token that all heads share (a latent vector from which keys and values are
+    expanded, with whatever else the scores need), in pages; ``window`` as for ``PagedKV``: the LARGEST window among
+    the layers that read the rows.  Device layout per group of ``n`` layers: ``[n, pages, page, width]`` in the
+    activation dtype; a token's row is contiguous."""
+
+    width: int
+    window: Optional[int] = None
+    paged = True
+
+    def page_bytes(self, page_size, act_dtype):
+        return self.width * page_size * _elem(act_dtype)
+
+    def allocate(self, num_layers, count, page_size, act_dtype, device):
+        return [torch.zeros((num_layers, count, page_size, self.width), dtype=act_dtype, device=device)]
+
+    def layer_view(self, group, tensors, index, page_size):
+        return PagedRowsLayer(group, tensors[0][index], page_size)
+
+
+@dataclasses.dataclass(frozen=True)
 class FixedState(CacheKind):
     """State of fixed size per request, ``shape`` elements of ``dtype``
-    ("float32" or "activation") in a slot; zeroed when a request runs its first tokens.
+    ("float32", "int32" or "activation") in a slot; zeroed when a request runs its first tokens.
     Device layout per group of ``n`` layers: ``[n, slots, *shape]``."""
 
     shape: Tuple[int, ...]
@@ -101,7 +130,7 @@ class FixedState(CacheKind):
     paged = False
 
     def _dtype(self, act_dtype):
-        return torch.float32 if self.dtype == "float32" else act_dtype
+        return {"float32": torch.float32, "int32": torch.int32}.get(self.dtype, act_dtype)
 
     def page_bytes(self, page_size, act_dtype):
         n = 1

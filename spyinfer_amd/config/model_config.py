@@ -164,3 +164,125 @@ class Qwen3Config(ModelConfig):
         if raw.get("use_sliding_window"):
             raise ConfigError("config.json: use_sliding_window is set, but this architecture attends to all keys "
                               "(src/backends/cpu/cpu_attention.cpp:98-111)")
+
+
+def _need(raw: Dict[str, Any], path: str, kinds, where: str = "config.json"):
+    """raw[a][b][c] for path "a.b.c", checked for presence and type."""
+    node = raw
+    for key in path.split("."):
+        if not isinstance(node, dict) or key not in node or node[key] is None:
+            raise ConfigError("%s lacks %r" % (where, path))
+        node = node[key]
+    if isinstance(node, bool) or not isinstance(node, kinds):
+        raise ConfigError("%s: %r has value %r of the wrong type" % (where, path, node))
+    return node
+
+
+@dataclasses.dataclass
+class SefevikConfig(ModelConfig):
+    """Sefevik: layers that add the norm of a sublayer's output to the stream and hand on a learned mix of all layer
+    results so far; token mixers 'mingru' (a gated recurrence) and 'latent_attention' (keys and values expanded from a
+    low-rank vector per token, rotated shared key part, window, sink); an embedding with a hashed pair table.  The
+    configuration is nested; ``layers`` lists every layer's type and sizes, and nothing is assumed equal between
+    layers."""
+
+    architecture: str = ""
+    vocab: int = -1
+    width: int = -1
+    norm_eps: float = 0.0
+    #: pair table of the embedding: rows (without the first-token row), multipliers of the previous and the current id;
+    #: buckets == 0: the model has none
+    bigram_buckets: int = 0
+    bigram_mul_prev: int = 0
+    bigram_mul_cur: int = 0
+    #: one dict per layer: type, mixer (sizes and constants of that mixer), mlp (None or {kind, ff})
+    layers: List[Dict[str, Any]] = dataclasses.field(default_factory=list)
+
+    MIXERS: ClassVar[tuple] = ("mingru", "latent_attention")
+
+    @classmethod
+    def from_dict(cls, raw: Dict[str, Any]) -> "SefevikConfig":
+        cfg = cls(architecture=str(raw.get("architecture") or (raw.get("architectures") or [""])[0]),
+                  vocab=_need(raw, "vocab", int), width=_need(raw, "width", int), norm_eps=float(_need(raw, "norm.eps", (int, float))))
+        pair = (raw.get("embedding") or {}).get("bigram")
+        if pair:
+            cfg.bigram_buckets = _need(pair, "buckets", int, "config.json embedding.bigram")
+            cfg.bigram_mul_prev = _need(pair, "mul_prev", int, "config.json embedding.bigram")
+            cfg.bigram_mul_cur = _need(pair, "mul_cur", int, "config.json embedding.bigram")
+        layers = _need(raw, "layers", list)
+        cfg.layers = [cls._layer(i, l) for i, l in enumerate(layers)]
+        cfg._raw = dict(raw)
+        cfg.validate()
+        return cfg
+
+    @classmethod
+    def _layer(cls, i: int, raw: Dict[str, Any]) -> Dict[str, Any]:
+        where = "config.json layers[%d]" % i
+        if not isinstance(raw, dict):
+            raise ConfigError("%s is no object" % where)
+        kind = _need(raw, "type", str, where)
+        if kind not in cls.MIXERS:
+            raise ConfigError("%s: mixer type %r is not known (%s)" % (where, kind, ", ".join(cls.MIXERS)))
+        m = _need(raw, "mixer", dict, where)
+        out = {"type": kind, "mlp": None}
+        if kind == "mingru":
+            out["mixer"] = {"width": _need(m, "width", int, where + ".mixer")}
+        else:
+            mix = {k: _need(m, k, int, where + ".mixer") for k in ("heads", "dim", "rot_dim", "vdim", "kv_rank")}
+            mix["scale"] = float(_need(m, "scale", (int, float), where + ".mixer"))
+            mix["kv_from"] = _need(m, "kv_from", int, where + ".mixer") if m.get("kv_from") is not None else None
+            mix["window"] = _need(m, "mask.size", int, where + ".mixer") if m.get("mask") else None
+            rot = m.get("rot")
+            if rot:
+                mix["rot"] = {"base": float(_need(rot, "base", (int, float), where + ".mixer.rot")),
+                              "dims": _need(rot, "dims", int, where + ".mixer.rot") if rot.get("dims") is not None else mix["rot_dim"],
+                              "scaling": None}
+                sc = rot.get("scaling")
+                if sc:
+                    mix["rot"]["scaling"] = {k: float(_need(sc, k, (int, float), where + ".mixer.rot.scaling"))
+                                             for k in ("factor", "original", "fast", "slow")}
+            else:
+                mix["rot"] = None
+            out["mixer"] = mix
+        mlp = raw.get("mlp")
+        if mlp is not None:
+            kind = _need(mlp, "kind", str, where + ".mlp")
+            if kind != "dense":
+                raise ConfigError("%s.mlp: kind %r is not known (dense)" % (where, kind))
+            out["mlp"] = {"kind": kind, "ff": _need(mlp, "ff", int, where + ".mlp")}
+        return out
+
+    def to_dict(self) -> Dict[str, Any]:
+        return dict(getattr(self, "_raw", {}))
+
+    def validate(self) -> None:
+        if self.vocab <= 0 or self.width <= 0:
+            raise ConfigError("config.json: vocab and width must be positive")
+        if not (self.norm_eps > 0.0):
+            raise ConfigError("config.json: norm.eps must be positive")
+        if self.bigram_buckets < 0:
+            raise ConfigError("config.json: embedding.bigram.buckets must be positive")
+        if not self.layers:
+            raise ConfigError("config.json: no layers")
+        for i, layer in enumerate(self.layers):
+            m = layer["mixer"]
+            if any(isinstance(v, int) and not isinstance(v, bool) and v <= 0 for k, v in m.items() if k not in ("kv_from", "dim")):
+                raise ConfigError("config.json layers[%d].mixer: sizes must be positive" % i)
+            if layer["mlp"] and layer["mlp"]["ff"] <= 0:
+                raise ConfigError("config.json layers[%d].mlp.ff must be positive" % i)
+            if layer["type"] != "latent_attention":
+                continue
+            if m["dim"] < 0:
+                raise ConfigError("config.json layers[%d].mixer.dim must not be negative" % i)
+            rot = m["rot"]
+            if rot and (rot["dims"] % 2 or not (0 < rot["dims"] <= m["rot_dim"]) or not rot["base"] > 1.0):
+                raise ConfigError("config.json layers[%d].mixer.rot: dims must be even and at most rot_dim, base above 1" % i)
+            src = m["kv_from"]
+            if src is not None:
+                if not (0 <= src < i) or self.layers[src]["type"] != "latent_attention" or self.layers[src]["mixer"]["kv_from"] is not None:
+                    raise ConfigError("config.json layers[%d].mixer.kv_from = %r must name an earlier latent_attention layer "
+                                      "with a projection of its own" % (i, src))
+                other = self.layers[src]["mixer"]
+                if (other["kv_rank"], other["rot_dim"], other["rot"]) != (m["kv_rank"], m["rot_dim"], m["rot"]):
+                    raise ConfigError("config.json layers[%d].mixer: kv_rank, rot_dim and rot must equal those of layer %d, "
+                                      "whose cache it reads" % (i, src))

@@ -44,8 +44,11 @@ def get_architecture(name: str) -> Architecture:
 
 def architecture_of(raw: dict) -> Architecture:
     archs = raw.get("architectures")
+    if archs is None and isinstance(raw.get("architecture"), str):
+        archs = [raw["architecture"]]            # some configurations name their one architecture as a string
     if not isinstance(archs, list) or not archs or not isinstance(archs[0], str):
-        raise ConfigError("config.json lacks 'architectures': [name]; known: %s" % ", ".join(registered_architectures()))
+        raise ConfigError("config.json lacks 'architectures': [name] (or 'architecture': name); known: %s"
+                          % ", ".join(registered_architectures()))
     return get_architecture(archs[0])
 
 

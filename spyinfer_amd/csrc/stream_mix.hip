@@ -1,0 +1,164 @@
+// Operations on the float32 residual stream for layers that norm a sublayer's OUTPUT and for models that mix the
+// results of earlier layers: an embedding with a hashed pair table, stream + norm(y), a weighted sum of kept layer
+// results, and the xIELU activation.  All arithmetic is float32; a bfloat16 value is rounded once, when it is written.
+#include "common.h"
+#include <math.h>
+
+// ---------------------------------------------------------------------------------------------
+// out[t] = table[id[t]] + pair[row(t)], row = (prev * mul_prev + id * mul_cur) mod buckets, the last row (number
+// `buckets`) for a request's first token.  prev is the token before in the step, or for an entry's first token the one
+// that the request's state slot holds (`last_token`, written by the steps before).  copy (optional): the same values in
+// the activation dtype, for the products that read the stream.
+template <typename TW, typename TA>
+__global__ void pair_embedding_kernel(float* __restrict__ out, TA* __restrict__ copy, const TW* __restrict__ table,
+                                      const TW* __restrict__ pair, const int* __restrict__ ids, const int* __restrict__ positions,
+                                      const int* __restrict__ token_entry, const int* __restrict__ cu_q,
+                                      const int* __restrict__ slot_ids, const int* __restrict__ last_token, int num_slots,
+                                      int H, int V, int buckets, long long mul_prev, long long mul_cur) {
+    const int t = blockIdx.x;
+    const int id = ids[t];
+    float* o = out + (size_t)t * H;
+    TA* c = copy ? copy + (size_t)t * H : nullptr;
+    if (id < 0 || id >= V) {
+        for (int i = threadIdx.x; i < H; i += blockDim.x) { o[i] = 0.f; if (c) c[i] = from_f32<TA>(0.f); }
+        return;
+    }
+    const TW* row = table + (size_t)id * H;
+    const TW* prow = nullptr;
+    if (pair) {
+        int r = buckets;
+        if (positions[t] > 0) {
+            const int e = token_entry[t];
+            int prev;
+            if (t == cu_q[e]) {
+                const int slot = slot_ids[e];
+                prev = (slot >= 0 && slot < num_slots) ? last_token[slot] : 0;
+            } else {
+                prev = ids[t - 1];
+            }
+            long long h = ((long long)prev * mul_prev + (long long)id * mul_cur) % (long long)buckets;
+            if (h < 0) h += buckets;
+            r = (int)h;
+        }
+        prow = pair + (size_t)r * H;
+    }
+    for (int i = threadIdx.x; i < H; i += blockDim.x) {
+        float v = to_f32<TW>(row[i]);
+        if (prow) v += to_f32<TW>(prow[i]);
+        o[i] = v;
+        if (c) c[i] = from_f32<TA>(v);
+    }
+}
+
+// last_token[slot of entry e] = the entry's last token of this step (after every block above has read the old value:
+// it is a launch of its own)
+__global__ void keep_last_token_kernel(int* __restrict__ last_token, const int* __restrict__ ids, const int* __restrict__ cu_q,
+                                       const int* __restrict__ slot_ids, int S, int num_slots) {
+    const int e = blockIdx.x * blockDim.x + threadIdx.x;
+    if (e >= S) return;
+    const int slot = slot_ids[e];
+    const int n = cu_q[e + 1];
+    if (slot >= 0 && slot < num_slots && n > cu_q[e]) last_token[slot] = ids[n - 1];
+}
+
+extern "C" int spy_pair_embedding(float* out, void* copy, int copy_dtype, const void* table, const void* pair, int table_dtype,
+                                  const int* ids, const int* positions, const int* token_entry, const int* cu_q,
+                                  const int* slot_ids, int* last_token, int num_slots, int S, int T, int H, int V, int buckets,
+                                  long long mul_prev, long long mul_cur, hipStream_t st) {
+    SPY_REQUIRE(T > 0 && S > 0 && H > 0 && V > 0, "spy_pair_embedding: empty operand");
+    SPY_REQUIRE(!pair || (buckets > 0 && last_token && num_slots > 0), "spy_pair_embedding: a pair table needs buckets and the slots' last tokens");
+    const int threads = H >= 1024 ? 256 : 64;
+    SPY_DISPATCH(table_dtype, TW, SPY_DISPATCH(copy_dtype, TA, (pair_embedding_kernel<TW, TA><<<T, threads, 0, st>>>(
+        out, (TA*)copy, (const TW*)table, (const TW*)pair, ids, positions, token_entry, cu_q, slot_ids, last_token, num_slots, H, V,
+        buckets, mul_prev, mul_cur))));
+    SPY_CHECK_LAUNCH("spy_pair_embedding");
+    if (pair) {
+        keep_last_token_kernel<<<(S + 63) / 64, 64, 0, st>>>(last_token, ids, cu_q, slot_ids, S, num_slots);
+        SPY_CHECK_LAUNCH("spy_pair_embedding (last tokens)");
+    }
+    return 0;
+}
+
+// ---------------------------------------------------------------------------------------------
+// out[t] = base[t] + y[t] / sqrt(mean(y[t]^2) + eps) * w;  copy[t] (optional) = the same in the activation dtype.
+// out may be base (in place).  One block per row; y is read twice (the second read comes from the cache).
+template <typename TY, typename TW, typename TA>
+__global__ void norm_residual_kernel(float* __restrict__ out, TA* __restrict__ copy, const float* __restrict__ base,
+                                     const TY* __restrict__ y, const TW* __restrict__ w, float eps, int H) {
+    __shared__ float red[16];
+    const size_t off = (size_t)blockIdx.x * H;
+    const TY* yr = y + off;
+    float ss = 0.f;
+    for (int i = threadIdx.x; i < H; i += blockDim.x) { const float v = to_f32<TY>(yr[i]); ss += v * v; }
+    ss = block_sum(ss, red);
+    const float scale = 1.0f / sqrtf(ss / (float)H + eps);
+    for (int i = threadIdx.x; i < H; i += blockDim.x) {
+        const float v = base[off + i] + (scale * to_f32<TY>(yr[i])) * to_f32<TW>(w[i]);
+        out[off + i] = v;
+        if (copy) copy[off + i] = from_f32<TA>(v);
+    }
+}
+
+extern "C" int spy_norm_residual(float* out, void* copy, int copy_dtype, const float* base, const void* y, int y_dtype,
+                                 const void* w, int w_dtype, float eps, int T, int H, hipStream_t st) {
+    SPY_REQUIRE(T > 0 && H > 0, "spy_norm_residual: empty operand");
+    const int threads = H >= 2048 ? 512 : (H >= 512 ? 256 : 64);
+    SPY_DISPATCH(y_dtype, TY, SPY_DISPATCH(w_dtype, TW, SPY_DISPATCH(copy_dtype, TA, (norm_residual_kernel<TY, TW, TA><<<T, threads, 0, st>>>(
+        out, (TA*)copy, base, (const TY*)y, (const TW*)w, eps, H)))));
+    SPY_CHECK_LAUNCH("spy_norm_residual");
+    return 0;
+}
+
+// ---------------------------------------------------------------------------------------------
+// out[i] = sum over j < n of a[j] * kept[j][i], added in ascending j; kept is [n or more][count] float32 with `stride`
+// elements between layers.  copy (optional): the result in the activation dtype.
+#define DEPTH_MAX 256
+template <typename TW, typename TA>
+__global__ void depth_mix_kernel(float* __restrict__ out, TA* __restrict__ copy, const float* __restrict__ kept, size_t stride,
+                                 const TW* __restrict__ a, int n, size_t count) {
+    __shared__ float as[DEPTH_MAX];
+    for (int j = threadIdx.x; j < n; j += blockDim.x) as[j] = to_f32<TW>(a[j]);
+    __syncthreads();
+    for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < count; i += (size_t)gridDim.x * blockDim.x) {
+        float s = 0.f;
+        for (int j = 0; j < n; ++j) s = fmaf(as[j], kept[(size_t)j * stride + i], s);
+        out[i] = s;
+        if (copy) copy[i] = from_f32<TA>(s);
+    }
+}
+
+extern "C" int spy_depth_mix(float* out, void* copy, int copy_dtype, const float* kept, long long stride, const void* a, int a_dtype,
+                             int n, long long count, hipStream_t st) {
+    SPY_REQUIRE(n > 0 && n <= DEPTH_MAX && count > 0 && stride >= count, "spy_depth_mix: %d layers (1..%d allowed), %lld values", n, DEPTH_MAX, count);
+    long long blocks = (count + 255) / 256;
+    if (blocks > 8192) blocks = 8192;
+    SPY_DISPATCH(a_dtype, TW, SPY_DISPATCH(copy_dtype, TA, (depth_mix_kernel<TW, TA><<<(unsigned)blocks, 256, 0, st>>>(
+        out, (TA*)copy, kept, (size_t)stride, (const TW*)a, n, (size_t)count))));
+    SPY_CHECK_LAUNCH("spy_depth_mix");
+    return 0;
+}
+
+// ---------------------------------------------------------------------------------------------
+// xIELU with the two learned numbers pq = (p, q):  z > 0: softplus(p) z^2 + z/2;  z <= 0: (1/2 + softplus(q)) (e^z - 1 - z) + z/2
+__device__ __forceinline__ float softplus_f(float x) { return fmaxf(x, 0.f) + log1pf(expf(-fabsf(x))); }
+
+__device__ __forceinline__ float xielu_f(float z, float ap, float aq) {
+    return z > 0.f ? fmaf(ap * z, z, 0.5f * z) : fmaf(aq, expm1f(z) - z, 0.5f * z);
+}
+
+template <typename TA, typename TW>
+__global__ void xielu_kernel(TA* __restrict__ out, const TA* __restrict__ in, const TW* __restrict__ pq, size_t count) {
+    const float ap = softplus_f(to_f32<TW>(pq[0])), aq = 0.5f + softplus_f(to_f32<TW>(pq[1]));
+    for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < count; i += (size_t)gridDim.x * blockDim.x)
+        out[i] = from_f32<TA>(xielu_f(to_f32<TA>(in[i]), ap, aq));
+}
+
+extern "C" int spy_xielu(void* out, const void* in, int dtype, const void* pq, int pq_dtype, long long count, hipStream_t st) {
+    SPY_REQUIRE(count > 0, "spy_xielu: empty operand");
+    long long blocks = (count + 255) / 256;
+    if (blocks > 8192) blocks = 8192;
+    SPY_DISPATCH(dtype, TA, SPY_DISPATCH(pq_dtype, TW, (xielu_kernel<TA, TW><<<(unsigned)blocks, 256, 0, st>>>(
+        (TA*)out, (const TA*)in, (const TW*)pq, (size_t)count))));
+    SPY_CHECK_LAUNCH("spy_xielu");
+    return 0;
+}

@@ -39,7 +39,7 @@ def run(argv=None, stdin=None, stdout=None) -> int:
     ap.add_argument("--max-tokens", type=int, required=True,
                     help="most tokens that live requests hold at any time (each rounded up to a multiple of 64)")
     ap.add_argument("--kvcache-block-size", type=int, default=16, help="tokens in a cache page")
-    ap.add_argument("--max-num-seqs", type=int, default=8, help="most live requests")
+    ap.add_argument("--max-num-seqs", type=int, default=4, help="most live requests (state slots)")
     ap.add_argument("--device", default="cuda:0")
     ap.add_argument("--poison-cache", action="store_true",
                     help="fill the cache pool with NaN before the first step: a read of a slot that no step wrote shows in the logits")

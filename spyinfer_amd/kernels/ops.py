@@ -74,7 +74,9 @@ class _Hip:
                      "spy_attention_generic", "spy_attention_mfma", "spy_attention_mfma_workspace", "spy_attention_mfma_part_workspace", "spy_attention_prefill",
                      "spy_attention_prefill_workspace", "spy_swiglu", "spy_untile_weight",
                      "spy_sample", "spy_sample_workspace", "spy_gemm_skinny", "spy_gemm_skinny_swiglu",
-                     "spy_gemm_decode", "spy_gemm_decode_workspace", "spy_embedding_sumsq", "spy_sample_static", "spy_measure_read"):
+                     "spy_gemm_decode", "spy_gemm_decode_workspace", "spy_embedding_sumsq", "spy_sample_static", "spy_measure_read",
+                     "spy_pair_embedding", "spy_norm_residual", "spy_depth_mix", "spy_xielu", "spy_mingru", "spy_latent_prepare",
+                     "spy_gemm_strided", "spy_latent_attention"):
             if not hasattr(self.lib, name):
                 raise KernelError("the kernel library %s lacks %s: it is older than its sources; build it again "
                                   "(spyinfer_amd.kernels.build.build())" % (self.lib._name, name))
@@ -842,6 +844,191 @@ def sample(logits: torch.Tensor, temperature: torch.Tensor, u: torch.Tensor) -> 
         ws = torch.empty((hip().lib.spy_sample_workspace(ctypes.c_int(R)),), dtype=torch.float32, device=logits.device)
         hip().call("spy_sample", _ptr(logits), _ptr(temperature), _ptr(u), _ptr(out), ctypes.c_int(R), ctypes.c_int(V),
                    _ptr(ws), _Hip.stream())
+    return out
+
+
+# --------------------------------------------------------------------------
+# The stream of layers that norm a sublayer's output, kept layer results, and their activation
+def _copy_of(like: torch.Tensor, copy_dtype: Optional[torch.dtype]):
+    """The activation-dtype copy that a stream kernel writes beside its float32 result (None where the activations are
+    float32 themselves: the result serves)."""
+    if copy_dtype is None or copy_dtype == torch.float32:
+        return None
+    _check(copy_dtype == torch.bfloat16, "a copy of the stream is bfloat16 or float32")
+    return torch.empty(like.shape, dtype=copy_dtype, device=like.device)
+
+
+def pair_embedding(ids: torch.Tensor, table: torch.Tensor, pair: Optional[torch.Tensor], buckets: int, mul_prev: int, mul_cur: int,
+                   positions: torch.Tensor, token_entry: torch.Tensor, cu_q: torch.Tensor, slot_ids: torch.Tensor,
+                   last_token: Optional[torch.Tensor], copy_dtype: Optional[torch.dtype] = None):
+    """out[t] = table[ids[t]] + pair[(prev * mul_prev + ids[t] * mul_cur) mod buckets] in float32, row ``buckets`` of
+    ``pair`` for a request's first token; prev is the token before, inside the step or, for an entry's first token, in
+    ``last_token[slot]`` (int32 [slots]), where every entry's last token is left afterwards.  Returns (out [T, H]
+    float32, copy in ``copy_dtype`` or None)."""
+    _dev(ids, table, pair, positions, token_entry, cu_q, slot_ids, last_token)
+    _check(ids.dtype == torch.int32 and ids.dim() == 1, "pair_embedding: ids must be int32 [T]")
+    _check(table.dim() == 2, "pair_embedding: table must be [V, H]")
+    T, (V, H), S = ids.shape[0], table.shape, slot_ids.shape[0]
+    for name, arr, n in (("positions", positions, T), ("token_entry", token_entry, T), ("cu_q", cu_q, S + 1), ("slot_ids", slot_ids, S)):
+        _check(arr.dtype == torch.int32 and tuple(arr.shape) == (n,), "pair_embedding: %s must be int32 [%d]", name, n)
+    if pair is not None:
+        _check(pair.dtype == table.dtype and tuple(pair.shape) == (buckets + 1, H) and buckets > 0,
+               "pair_embedding: the pair table must be [buckets + 1, H] of the table's dtype")
+        _check(last_token is not None and last_token.dtype == torch.int32 and last_token.dim() == 1,
+               "pair_embedding: the slots' last tokens must be int32 [slots]")
+    out = torch.empty((T, H), dtype=torch.float32, device=table.device)
+    copy = _copy_of(out, copy_dtype)
+    if T:
+        hip().call("spy_pair_embedding", _ptr(out), _ptr(copy), BF16 if copy is not None else F32, _ptr(table), _ptr(pair),
+                   _code(table, "embedding table"), _ptr(ids), _ptr(positions), _ptr(token_entry), _ptr(cu_q), _ptr(slot_ids),
+                   _ptr(last_token), ctypes.c_int(0 if last_token is None else last_token.shape[0]), ctypes.c_int(S),
+                   ctypes.c_int(T), ctypes.c_int(H), ctypes.c_int(V), ctypes.c_int(buckets), ctypes.c_longlong(mul_prev),
+                   ctypes.c_longlong(mul_cur), _Hip.stream())
+    return out, copy
+
+
+def norm_residual(base: torch.Tensor, y: torch.Tensor, weight: torch.Tensor, eps: float, out: Optional[torch.Tensor] = None,
+                  copy_dtype: Optional[torch.dtype] = None):
+    """out = base + y / sqrt(mean(y^2) + eps) * weight, float32 (``out`` may be ``base``; a new tensor if None).
+    Returns (out, copy of out in ``copy_dtype`` or None)."""
+    _dev(base, y, weight, out)
+    _check(base.dtype == torch.float32 and base.dim() == 2, "norm_residual: the stream must be float32 [T, H]")
+    T, H = base.shape
+    _check(tuple(y.shape) == (T, H) and weight.shape == (H,), "norm_residual: y [T, H] and weight [H] expected")
+    if out is None:
+        out = torch.empty_like(base)
+    _check(out.dtype == torch.float32 and tuple(out.shape) == (T, H), "norm_residual: out must be float32 [T, H]")
+    copy = _copy_of(out, copy_dtype)
+    if T:
+        hip().call("spy_norm_residual", _ptr(out), _ptr(copy), BF16 if copy is not None else F32, _ptr(base), _ptr(y), _code(y, "y"),
+                   _ptr(weight), _code(weight, "norm weight"), ctypes.c_float(eps), ctypes.c_int(T), ctypes.c_int(H), _Hip.stream())
+    return out, copy
+
+
+def depth_mix(kept: torch.Tensor, n: int, a: torch.Tensor, copy_dtype: Optional[torch.dtype] = None):
+    """sum over j < n of a[j] * kept[j] for ``kept [layers, T, H]`` float32, added in ascending j.  Returns (float32
+    [T, H], copy in ``copy_dtype`` or None)."""
+    _dev(kept, a)
+    _check(kept.dtype == torch.float32 and kept.dim() == 3 and 0 < n <= kept.shape[0], "depth_mix: kept must be float32 [layers >= n, T, H]")
+    _check(a.dim() == 1 and a.shape[0] == n, "depth_mix: one weight per kept layer expected")
+    out = torch.empty(kept.shape[1:], dtype=torch.float32, device=kept.device)
+    copy = _copy_of(out, copy_dtype)
+    if out.numel():
+        hip().call("spy_depth_mix", _ptr(out), _ptr(copy), BF16 if copy is not None else F32, _ptr(kept), ctypes.c_longlong(out.numel()),
+                   _ptr(a), _code(a, "depth weights"), ctypes.c_int(n), ctypes.c_longlong(out.numel()), _Hip.stream())
+    return out, copy
+
+
+def xielu(x: torch.Tensor, pq: torch.Tensor) -> torch.Tensor:
+    """In place: x > 0: softplus(p) x^2 + x/2; x <= 0: (1/2 + softplus(q)) (e^x - 1 - x) + x/2, with pq = (p, q) on the device."""
+    _dev(x, pq)
+    _check(pq.numel() == 2, "xielu: two numbers (p, q) expected")
+    if x.numel():
+        hip().call("spy_xielu", _ptr(x), _ptr(x), _code(x, "x"), _ptr(pq), _code(pq, "xielu numbers"), ctypes.c_longlong(x.numel()),
+                   _Hip.stream())
+    return x
+
+
+def linear_xielu(x: torch.Tensor, w: torch.Tensor, pq: torch.Tensor, tiled: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """xielu(x . w^T)."""
+    return xielu(linear(x, w, tiled=tiled), pq)
+
+
+# --------------------------------------------------------------------------
+def mingru(zxg: torch.Tensor, bz: torch.Tensor, bx: torch.Tensor, state: torch.Tensor, pieces: torch.Tensor, n_pieces: int,
+           multi: bool, slot_ids: torch.Tensor) -> torch.Tensor:
+    """The minGRU recurrence over the step's tokens.  ``zxg [T, 3 W]`` = the projections [z | x | g] of every token;
+    S = (1 - z) S + z c with z = sigmoid(. + bz), c from x + bx; ``state [slots, W]`` float32 is read at an entry's
+    start and left at its end.  ``pieces`` int32 [4 n]: entry, first row, end row and the entry's first piece, for
+    every piece of tokens (an entry in several pieces is walked by several blocks; ``multi`` says there is one).
+    Returns S_t * silu(g_t), [T, W] in the dtype of ``zxg``."""
+    _dev(zxg, bz, bx, state, pieces, slot_ids)
+    _check(zxg.dim() == 2 and zxg.shape[1] % 3 == 0, "mingru: projections [T, 3 W] expected")
+    T, W = zxg.shape[0], zxg.shape[1] // 3
+    _check(bz.shape == (W,) and bx.shape == (W,) and bz.dtype == bx.dtype, "mingru: two biases [W] of one dtype expected")
+    _check(state.dtype == torch.float32 and state.dim() == 2 and state.shape[1] == W, "mingru: state must be float32 [slots, W]")
+    _check(pieces.dtype == torch.int32 and pieces.shape == (4 * n_pieces,) and slot_ids.dtype == torch.int32,
+           "mingru: pieces must be int32 [4 n] and slot_ids int32")
+    out = torch.empty((T, W), dtype=zxg.dtype, device=zxg.device)
+    if T:
+        ab = torch.empty((n_pieces, 2, W), dtype=torch.float32, device=zxg.device) if multi else None
+        hip().call("spy_mingru", _ptr(out), _ptr(state), _ptr(ab), _ptr(zxg), _code(zxg, "projections"), _ptr(bz), _ptr(bx),
+                   _code(bz, "biases"), _ptr(pieces), ctypes.c_int(n_pieces), ctypes.c_int(1 if multi else 0), _ptr(slot_ids),
+                   ctypes.c_int(state.shape[0]), ctypes.c_int(T), ctypes.c_int(W), _Hip.stream())
+    return out
+
+
+# --------------------------------------------------------------------------
+def gemm_strided(a: torch.Tensor, a_strides, b: torch.Tensor, b_strides, c: torch.Tensor, c_strides, batch: int, M: int, N: int,
+                 K: int) -> torch.Tensor:
+    """c[i][m][n] = sum_k a[i][m][k] * b[i][n][k] with element strides (batch, row, inner) for each operand, taken from
+    the tensors' first elements; float32 products and sums.  The caller answers for the strides staying inside the
+    tensors (checked here against their sizes)."""
+    _dev(a, b, c)
+    for t, (sb, sr, si), (nr, ni), name in ((a, a_strides, (M, K), "a"), (b, b_strides, (N, K), "b"), (c, c_strides, (M, N), "c")):
+        last = (batch - 1) * sb + (nr - 1) * sr + (ni - 1) * si
+        _check(min(sb, sr, si) >= 0 and last < t.numel(), "gemm_strided: the strides of %s reach beyond the tensor", name)
+    if batch * M * N:
+        hip().call("spy_gemm_strided", _ptr(a), _code(a, "a"), *(ctypes.c_longlong(s) for s in a_strides), _ptr(b), _code(b, "b"),
+                   *(ctypes.c_longlong(s) for s in b_strides), _ptr(c), _code(c, "c"), *(ctypes.c_longlong(s) for s in c_strides),
+                   ctypes.c_int(batch), ctypes.c_int(M), ctypes.c_int(N), ctypes.c_int(K), _Hip.stream())
+    return c
+
+
+def latent_prepare(q: torch.Tensor, dkv: Optional[torch.Tensor], cache: Optional[torch.Tensor], slot_mapping: Optional[torch.Tensor],
+                   w_norm: Optional[torch.Tensor], eps: float, freq: Optional[torch.Tensor], mag: float, dims: int,
+                   positions: torch.Tensor, H: int, DN: int, DR: int, R: int) -> torch.Tensor:
+    """Queries ``q [T, >= H (DN + DR)]`` (a row may be a view into a wider product: its stride is taken) and, if given,
+    ``dkv [T, >= R + DR]``: the latent rmsnorm(dkv[:R]) * w_norm and the rotated dkv[R:] go to ``cache [pages, P, R + DR]``
+    at the tokens' slots; returns the absorbed query rows float32 [T, H, R + DR] with the rotated part filled in (the
+    first R values of a row are for the caller's product with the keys' expansion matrix)."""
+    _check(q.dim() == 2 and q.stride(1) == 1 and q.is_cuda, "latent_prepare: q must be rows on the GPU")
+    T = q.shape[0]
+    _check(q.shape[1] >= H * (DN + DR), "latent_prepare: q rows hold %d values, %d heads of %d needed", q.shape[1], H, DN + DR)
+    _dev(cache, slot_mapping, w_norm, freq, positions)
+    _check(positions.dtype == torch.int32 and positions.shape == (T,), "latent_prepare: positions must be int32 [T]")
+    _check(dims == 0 or (freq is not None and freq.dtype == torch.float32 and freq.shape == (dims // 2,)),
+           "latent_prepare: one float32 frequency per rotated pair expected")
+    rows = 0
+    if dkv is not None:
+        _check(dkv.dim() == 2 and dkv.stride(1) == 1 and dkv.shape == (T, R + DR) and dkv.dtype == q.dtype and dkv.device == q.device,
+               "latent_prepare: dkv must be [T, R + DR] like q")
+        _check(cache is not None and cache.dtype == q.dtype and cache.dim() == 3 and cache.shape[2] == R + DR,
+               "latent_prepare: the cache must be [pages, P, R + DR] of the activation dtype")
+        _check(slot_mapping is not None and slot_mapping.dtype == torch.int32 and slot_mapping.shape == (T,) and w_norm is not None
+               and w_norm.shape == (R,), "latent_prepare: slot_mapping int32 [T] and a norm weight [R] expected")
+        rows = cache.shape[0] * cache.shape[1]
+    qa = torch.empty((T, H, R + DR), dtype=torch.float32, device=q.device)
+    if T:
+        hip().call("spy_latent_prepare", _ptr(qa), ctypes.c_void_p(q.data_ptr()), ctypes.c_int(q.stride(0)),
+                   ctypes.c_void_p(0 if dkv is None else dkv.data_ptr()), ctypes.c_int(0 if dkv is None else dkv.stride(0)),
+                   _code(q, "q"), _ptr(cache if dkv is not None else None), _ptr(slot_mapping if dkv is not None else None),
+                   ctypes.c_longlong(rows), _ptr(w_norm if dkv is not None else None),
+                   _code(w_norm, "norm weight") if dkv is not None else F32, ctypes.c_float(eps), _ptr(freq), ctypes.c_float(mag),
+                   ctypes.c_int(dims), _ptr(positions), ctypes.c_int(T), ctypes.c_int(H), ctypes.c_int(DN), ctypes.c_int(DR),
+                   ctypes.c_int(R), _Hip.stream())
+    return qa
+
+
+def latent_attention(qa: torch.Tensor, cache: torch.Tensor, page_size: int, meta: "AttentionMeta", sink: Optional[torch.Tensor],
+                     R: int, scale: float, window: Optional[int], out_dtype: torch.dtype) -> torch.Tensor:
+    """Attention of ``qa [T, H, R + DR]`` (float32, absorbed queries) over the latent rows ``cache [pages, P, R + DR]``:
+    score = qa . row * scale, softmax with exp(sink[h]) added to the denominator, causal with ``window``; the result is
+    sum_j p_j row_j[:R], [T, H, R] in ``out_dtype``."""
+    _dev(qa, cache, sink, meta.kv_len, meta.block_table, meta.token_entry, meta.positions)
+    _check(qa.dtype == torch.float32 and qa.dim() == 3, "latent_attention: qa must be float32 [T, H, D]")
+    T, H, D = qa.shape
+    _check(T == meta.T and cache.dim() == 3 and cache.shape[1] == page_size and cache.shape[2] == D and 0 < R <= D,
+           "latent_attention: cache [pages, P, %d] expected for %d tokens", D, meta.T)
+    _check(sink is None or sink.shape == (H,), "latent_attention: one sink per head expected")
+    _check(meta.block_table.shape == (meta.S, meta.max_blocks), "latent_attention: block table must be [S, max_blocks]")
+    out = torch.empty((T, H, R), dtype=out_dtype, device=qa.device)
+    if T:
+        hip().call("spy_latent_attention", _ptr(out), _code(out, "out"), _ptr(qa), _ptr(cache), _code(cache, "cache"),
+                   ctypes.c_int(page_size), ctypes.c_int(cache.shape[0]), _ptr(meta.kv_len), _ptr(meta.block_table),
+                   ctypes.c_int(meta.max_blocks), _ptr(meta.token_entry), _ptr(meta.positions), _ptr(sink),
+                   _code(sink, "sink") if sink is not None else F32, ctypes.c_int(meta.S), ctypes.c_int(T), ctypes.c_int(H),
+                   ctypes.c_int(R), ctypes.c_int(D - R), ctypes.c_float(scale), ctypes.c_int(int(window or 0)), _Hip.stream())
     return out
 
 

@@ -14,6 +14,7 @@ from typing import Dict, List, NamedTuple, Optional, Sequence
 import torch
 
 from ..parts.base import Block, Norm, PositionEncoding
+from ..parts.block import stream_copy
 from ..parts.embedding import LMHead, TokenEmbedding
 from ..weights.loader import WeightSpec
 
@@ -83,6 +84,12 @@ class DecoderModel:
                     raise ValueError("a call reads cache %d that no call writes" % call.cache)
                 if self.layers[call.layer].mixer.cache_spec() != specs[call.cache]:
                     raise ValueError("layer %d reads cache %d of another shape" % (call.layer, call.cache))
+        # an embedding that keeps something per request (the token before, say) has the cache id after the layers'
+        own = getattr(self.embed, "cache_spec", None)
+        self.embed_cache = None
+        if own is not None and own() is not None:
+            self.embed_cache = len(specs)
+            specs.append(own())
         return specs
 
     # ---- step ------------------------------------------------------------
@@ -109,7 +116,12 @@ class DecoderModel:
         at the batch's wanted rows (in ``logits_out`` if the caller brings a tensor of that shape)."""
         calls = self.schedule
         entry = [self.layers[c.layer].entry_norm() for c in calls] + [self.final_norm]
-        if self.position is None or type(self.position).on_embeddings is PositionEncoding.on_embeddings:
+        if hasattr(self.embed, "forward_step"):
+            # an embedding that reads more of the step than the token ids (and may keep state per request)
+            resid, copy = self.embed.forward_step(batch, storage.layer(self.embed_cache) if self.embed_cache is not None else None)
+            stream_copy(batch, resid, copy)
+            pending = None
+        elif self.position is None or type(self.position).on_embeddings is PositionEncoding.on_embeddings:
             resid, pending = self.embed.forward_for(batch.token_ids, entry[0], batch.act_dtype)
         else:
             resid, pending = self.position.on_embeddings(self.embed.forward(batch.token_ids), batch), None

@@ -51,6 +51,10 @@ class Norm(Part):
         the hidden state."""
         raise NotImplementedError
 
+    def add_normed(self, base: torch.Tensor, y: torch.Tensor, out: Optional[torch.Tensor] = None, copy_dtype=None):
+        """out = base + norm(y), float32, for blocks that norm a sublayer's output; (out, copy in ``copy_dtype`` or None)."""
+        raise NotImplementedError
+
     def foldable(self, out_dtype: torch.dtype):
         """None, or (weight, eps) if this norm can be folded into the products around it when a step has few rows:
         the product before it adds to the stream and prepares this norm's input, the product after it applies the

@@ -2,8 +2,11 @@
 The sums are carried as a pending addend and folded into the next norm's kernel."""
 from __future__ import annotations
 
+import torch
+
 from ..kernels import ops
-from .base import Block, FeedForward, Mixer, Norm
+from ..weights.loader import WeightSpec
+from .base import Block, FeedForward, Mixer, Norm, Part
 
 
 class PreNormBlock(Block):
@@ -52,3 +55,102 @@ class PreNormBlock(Block):
         a = self.mixer.forward(n1, batch, cache, store)
         n2 = self.norm2.add_norm(resid, a, act)
         return resid, self.ffn.forward(n2, batch)
+
+
+def stream_copy(batch, resid, copy=None):
+    """The residual stream in the activation dtype, for the products that read the stream itself.  A kernel that has
+    just written the stream leaves the copy here (``copy`` given); a reader asks for it (made now if nobody left one).
+    With float32 activations the stream serves."""
+    if resid.dtype == batch.act_dtype:
+        return resid
+    if copy is not None:
+        batch.shared["stream_copy"] = (resid, copy)
+        return copy
+    held = batch.shared.get("stream_copy")
+    if held is not None and held[0] is resid:
+        return held[1]
+    copy = resid.to(batch.act_dtype)
+    batch.shared["stream_copy"] = (resid, copy)
+    return copy
+
+
+class DepthMix(Part):
+    """What goes on to the next layer is a weighted sum of the results of all layers so far and of the embedding output:
+    x = sum_j a[j] X_j, j = 0 .. index + 1, with X_0 the embedding output and X_(j+1) the result of layer j (before any
+    such sum).  The step's results are kept in one float32 tensor [layers + 1, T, H], which the layers' results are
+    written into where they arise."""
+
+    def __init__(self, index: int, total: int, suffix: str = ""):
+        """``index``: the layer call this mix follows (0-based); ``total``: calls in the model's run order."""
+        self.index, self.total, self.suffix = index, total, suffix
+        self.weight = None
+
+    def weight_specs(self, prefix):
+        return [WeightSpec(prefix + self.suffix, (self.index + 2,), "mix")]
+
+    def bind(self, prefix, weights):
+        self.weight = weights[prefix + self.suffix]
+
+    def capturable(self, batch):
+        return True
+
+    def kept(self, batch, resid):
+        """The step's kept results; made when the first layer asks, with the stream as it stands as X_0."""
+        held = batch.shared.get("depth_kept")
+        if held is None:
+            held = torch.empty((self.total + 1,) + tuple(resid.shape), dtype=torch.float32, device=resid.device)
+            held[0].copy_(resid)
+            batch.shared["depth_kept"] = held
+        return held
+
+    def result_slot(self, batch, resid):
+        """Where this layer's result X_(index+1) is to be written."""
+        return self.kept(batch, resid)[self.index + 1]
+
+    def mix(self, batch):
+        """(the stream for the next layer, its copy in the activation dtype or None)."""
+        return ops.depth_mix(batch.shared["depth_kept"], self.index + 2, self.weight, batch.act_dtype)
+
+
+class OutputNormBlock(Block):
+    """h += norm1(mixer(h)); h += norm2(ffn(h)): the norm sits on a sublayer's OUTPUT, the sublayers read the stream
+    itself.  ``ffn`` (with ``norm2``) may be absent.  ``depth``: a ``DepthMix`` after the layer."""
+
+    def __init__(self, mixer: Mixer, norm1: Norm, ffn: FeedForward = None, norm2: Norm = None, depth: "DepthMix" = None,
+                 names=("mix", "norm1", "mlp", "norm2", "dwa")):
+        if (ffn is None) != (norm2 is None):
+            raise ValueError("a feed-forward and its norm come together")
+        self.mixer, self.norm1, self.ffn, self.norm2, self.depth = mixer, norm1, ffn, norm2, depth
+        self.names = names
+
+    def _parts(self, prefix):
+        parts = zip((self.mixer, self.norm1, self.ffn, self.norm2, self.depth), (prefix + "." + n for n in self.names))
+        return [(part, p) for part, p in parts if part is not None]
+
+    def weight_specs(self, prefix):
+        return [s for part, p in self._parts(prefix) for s in part.weight_specs(p)]
+
+    def bind(self, prefix, weights):
+        for part, p in self._parts(prefix):
+            part.bind(p, weights)
+
+    def capturable(self, batch):
+        return all(part.capturable(batch) for part, _ in self._parts(""))
+
+    def forward(self, resid, pending, batch, cache, store=True, next_norm=None):
+        act = batch.act_dtype
+        if pending is not None and not isinstance(pending, ops.ScaledInput):
+            resid.add_(pending.float())            # a block of another arrangement left an addend
+        x = stream_copy(batch, resid)
+        y = self.mixer.forward(x, batch, cache, store)
+        out = self.depth.result_slot(batch, resid) if self.depth is not None else resid
+        last = self.ffn is None
+        out, copy = self.norm1.add_normed(resid, y, out, None if (last and self.depth is not None) else act)
+        if not last:
+            x = stream_copy(batch, out, copy)
+            f = self.ffn.forward(x, batch)
+            out, copy = self.norm2.add_normed(out, f, out, None if self.depth is not None else act)
+        if self.depth is not None:
+            out, copy = self.depth.mix(batch)
+        stream_copy(batch, out, copy)
+        return out, None

@@ -36,26 +36,27 @@ class TokenEmbedding(Part):
 
 
 class LMHead(Part):
-    def __init__(self, vocab_size: int, hidden_size: int, tied_to: TokenEmbedding = None, fold_rows: int = 64):
+    def __init__(self, vocab_size: int, hidden_size: int, tied_to: TokenEmbedding = None, fold_rows: int = 64, suffix: str = ".weight"):
         """``fold_rows``: most rows for which the head runs as a decode product with the final norm folded in.  Above,
         the library's product after a norm kernel is faster for a large matrix (measured with 151936 x 4096: 235 / 246 /
         253 / 267 us at 24 / 32 / 48 / 64 rows against the library's 263 / 270 / 258 / 268 and a norm kernel of 6, but
         281 / 288 / 367 against 274 / 280 / 293 at 80 / 96 / 128)."""
         self.vocab_size, self.hidden_size, self.tied_to = vocab_size, hidden_size, tied_to
         self.fold_rows = fold_rows
+        self.suffix = suffix
         self.weight = None
 
     def weight_specs(self, prefix):
         if self.tied_to is not None:
             # a tied checkpoint may store the head again; it is not read (src/models/qwen3.hpp:46)
-            return [WeightSpec(prefix + ".weight", (self.vocab_size, self.hidden_size), optional=True)]
-        return [WeightSpec(prefix + ".weight", (self.vocab_size, self.hidden_size))]
+            return [WeightSpec(prefix + self.suffix, (self.vocab_size, self.hidden_size), optional=True)]
+        return [WeightSpec(prefix + self.suffix, (self.vocab_size, self.hidden_size))]
 
     def bind(self, prefix, weights):
         if self.tied_to is not None:
             self.weight, self.weight_tiled = ops.weight_forms(self.tied_to.weight, keep_rows=True)   # the table's rows are looked up
         else:
-            self.weight, self.weight_tiled = ops.weight_forms(weights.pop(prefix + ".weight"))
+            self.weight, self.weight_tiled = ops.weight_forms(weights.pop(prefix + self.suffix))
 
     def capturable(self, batch):
         return True
@@ -80,3 +81,43 @@ class LMHead(Part):
         if isinstance(normed, ops.ScaledInput):
             return ops.decode_linear(normed, self.weight_tiled, torch.float32, out)
         return ops.linear(normed, self.weight, torch.float32, tiled=self.weight_tiled, out=out)
+
+
+class PairHashEmbedding(TokenEmbedding):
+    """h[t] = E[id[t]] + B[row], row = (previous id * mul_prev + id[t] * mul_cur) mod buckets: a second table indexed by
+    a hash of the token and the one before it; a request's first token takes the table's last row (number ``buckets``).
+    The previous token of an entry's first token is part of the request's state: a slot of one int32
+    (``cache_spec``), which the step leaves at the entry's last token.  Without a pair table (``buckets`` = 0) it is a
+    plain embedding."""
+
+    def __init__(self, vocab_size: int, hidden_size: int, buckets: int = 0, mul_prev: int = 0, mul_cur: int = 0,
+                 names=("embed", "bigram")):
+        super().__init__(vocab_size, hidden_size)
+        self.buckets, self.mul_prev, self.mul_cur, self.names = int(buckets), int(mul_prev), int(mul_cur), names
+        self.pair = None
+
+    def weight_specs(self, prefix):
+        e, b = (prefix + n for n in self.names)
+        specs = [WeightSpec(e, (self.vocab_size, self.hidden_size))]
+        if self.buckets:
+            specs.append(WeightSpec(b, (self.buckets + 1, self.hidden_size)))
+        return specs
+
+    def bind(self, prefix, weights):
+        e, b = (prefix + n for n in self.names)
+        self.weight = weights[e]
+        if self.buckets:
+            self.pair = weights[b]
+            if self.pair.dtype != self.weight.dtype:
+                self.weight, self.pair = self.weight.float(), self.pair.float()
+
+    def cache_spec(self):
+        from ..cache.spec import FixedState
+        return FixedState((1,), "int32") if self.buckets else None
+
+    def forward_step(self, batch, cache):
+        """(stream float32 [T, H], its copy in the activation dtype or None) for the step's tokens."""
+        last = cache.state.view(-1) if cache is not None else None
+        return ops.pair_embedding(batch.token_ids, self.weight, self.pair, self.buckets, self.mul_prev, self.mul_cur,
+                                  batch.positions, batch.array("token_entry"), batch.array("cu_q"), batch.array("slot_ids"),
+                                  last, batch.act_dtype)

@@ -1,0 +1,114 @@
+"""Latent attention: keys and values of all heads are expanded from one low-rank vector per token.
+
+Per token the layer projects  q = Wq h  (per head ``dim`` unrotated and ``rot_dim`` rotated values) and
+d = Wdkv h  (``kv_rank + rot_dim`` values): c = rmsnorm(d[:kv_rank]) * w is the latent, d[kv_rank:] rotated is a key
+part that all heads share.  Head h has keys Wuk_h c and values Wuv_h c; its score against token j is
+(q_h[:dim] . Wuk_h c_j + rot(q_h[dim:]) . kr_j) * scale.  Only c and kr are cached, one row per token
+(``PagedRows``), and keys and values are never formed: the query is taken through Wuk_h once
+(qa_h = Wuk_h^T q_h[:dim], so that the score is qa_h . c_j + ...), the attention sums latents, and Wuv_h is applied to the
+sum.  Options: a sliding window (position i sees j with 0 <= i - j < window), a learned sink per head that adds
+exp(sink_h) to the softmax's denominator, and ``shares_cache``: the layer has no Wdkv and reads the rows of another
+layer (run order: ``LayerCall(layer, cache=that layer's, store=False)``).
+"""
+from __future__ import annotations
+
+from typing import Optional
+
+import torch
+
+from ..cache.spec import PagedRows
+from ..kernels import ops
+from ..weights.loader import WeightSpec
+from .attention import attention_meta
+from .base import Mixer
+from .rotary import RotaryEmbedding
+
+
+class LatentAttention(Mixer):
+    def __init__(self, hidden_size: int, heads: int, dim: int, rot_dim: int, vdim: int, kv_rank: int, scale: float, norm_eps: float,
+                 position: Optional[RotaryEmbedding] = None, window: Optional[int] = None, cache_window: Optional[int] = -1,
+                 sink: bool = True, shares_cache: bool = False,
+                 names=("q", "dkv", "dkv.norm", "uk", "uv", "sink", "o")):
+        """``window``: what this layer's queries see; ``cache_window``: what the cache rows are kept for, the largest
+        window of the layers that read them (None = everything; -1 = this layer's own window).  ``position``: a rotary
+        encoding over the rotated part (its ``rotary_dim`` <= rot_dim values are rotated)."""
+        self.hidden_size, self.heads, self.dim, self.rot_dim, self.vdim, self.kv_rank = hidden_size, heads, dim, rot_dim, vdim, kv_rank
+        self.scale, self.norm_eps = float(scale), float(norm_eps)
+        self.position, self.window = position, window
+        self.cache_window = window if cache_window == -1 else cache_window
+        if self.cache_window is not None and (window is None or window > self.cache_window):
+            raise ValueError("the cache rows are kept for %r tokens, the layer's window is %r" % (self.cache_window, window))
+        self.has_sink, self.shares_cache, self.names = sink, shares_cache, names
+        self.w_in = self.w_in_tiled = self.w_uk = self.w_uv = self.w_o = self.w_o_tiled = self.c_norm = self.sink = None
+
+    # ---- weights ---------------------------------------------------------
+    def _names(self, prefix):
+        return tuple(prefix + "." + n for n in self.names)
+
+    def weight_specs(self, prefix):
+        q, dkv, dkv_norm, uk, uv, sink, o = self._names(prefix)
+        H, nh, dn, dr, dv, r = self.hidden_size, self.heads, self.dim, self.rot_dim, self.vdim, self.kv_rank
+        specs = [WeightSpec(q, (nh * (dn + dr), H))]
+        if not self.shares_cache:
+            specs += [WeightSpec(dkv, (r + dr, H)), WeightSpec(dkv_norm, (r,), "norm")]
+        specs += [WeightSpec(uk, (nh * dn, r)), WeightSpec(uv, (nh * dv, r))]
+        if self.has_sink:
+            specs.append(WeightSpec(sink, (nh,), "bias"))
+        specs.append(WeightSpec(o, (H, nh * dv)))
+        return specs
+
+    def bind(self, prefix, weights):
+        q, dkv, dkv_norm, uk, uv, sink, o = self._names(prefix)
+        w_q = weights.pop(q)
+        if self.shares_cache:
+            w_in = w_q
+        else:
+            w_d = weights.pop(dkv)
+            if w_d.dtype != w_q.dtype:
+                w_q, w_d = w_q.float(), w_d.float()
+            w_in = torch.cat([w_q, w_d], dim=0).contiguous()          # one product: rows [q of all heads | dkv]
+            self.c_norm = weights[dkv_norm]
+        self.w_in, self.w_in_tiled = ops.weight_forms(w_in)
+        self.w_uk, self.w_uv = weights.pop(uk), weights.pop(uv)
+        self.w_o, self.w_o_tiled = ops.weight_forms(weights.pop(o))
+        if self.has_sink:
+            self.sink = weights[sink]
+        if self.position is not None:
+            self.position.prepare(self.w_uk.device, 0)
+
+    # ---- cache -----------------------------------------------------------
+    def cache_spec(self):
+        return PagedRows(self.kv_rank + self.rot_dim, self.cache_window)
+
+    def capturable(self, batch):
+        return True
+
+    def _frequencies(self):
+        if self.position is None:
+            return None, 1.0, 0
+        return self.position.frequencies()
+
+    # ---- step ------------------------------------------------------------
+    def forward(self, x, batch, cache, store=True):
+        if store == self.shares_cache:
+            raise ValueError("a latent attention layer %s" % ("without a projection of its own cannot fill a cache" if store
+                                                             else "with a projection of its own was told to read another's cache"))
+        nh, dn, dr, dv, r = self.heads, self.dim, self.rot_dim, self.vdim, self.kv_rank
+        T = x.shape[0]
+        qd = ops.linear(x, self.w_in, tiled=self.w_in_tiled)
+        nq = nh * (dn + dr)
+        freq, mag, dims = self._frequencies()
+        qa = ops.latent_prepare(qd, qd[:, nq:] if store else None, cache.rows if store else None,
+                                batch.slot_mapping(cache.group) if store else None, self.c_norm, self.norm_eps, freq, mag, dims,
+                                batch.positions, nh, dn, dr, r)
+        # the unrotated query parts through the keys' expansion: qa[t, h, :r] = sum_d q[t, h, d] Wuk[h dn + d, :]
+        if dn:
+            ops.gemm_strided(qd, (dn + dr, qd.stride(0), 1), self.w_uk, (dn * r, 1, r), qa, (r + dr, nh * (r + dr), 1), nh, T, r, dn)
+        else:
+            qa[:, :, :r].zero_()
+        meta = attention_meta(batch, cache.group, nh)
+        lat = ops.latent_attention(qa, cache.rows, cache.page_size, meta, self.sink, r, self.scale, self.window, x.dtype)
+        # the summed latents through the values' expansion: v[t, h, e] = sum_j lat[t, h, j] Wuv[h dv + e, j]
+        v = torch.empty((T, nh * dv), dtype=x.dtype, device=x.device)
+        ops.gemm_strided(lat, (r, nh * r, 1), self.w_uv, (dv * r, r, 1), v, (dv, nh * dv, 1), nh, T, dv, r)
+        return ops.linear(v, self.w_o, tiled=self.w_o_tiled)

@@ -52,3 +52,31 @@ class GatedMLP(FeedForward):
         weight, eps = next_norm.foldable(batch.act_dtype)
         return ops.decode_linear_residual(ops.decode_linear_swiglu(x, self.w_gate_up_tiled, for_product=True), self.w_down_tiled,
                                           resid, weight, eps, next_norm)
+
+
+class DenseMLP(FeedForward):
+    """down( act(up(x)) ), no gate and no biases.  ``activation`` "xielu": a piecewise activation with two learned
+    numbers (p, q) in a tensor of its own: z > 0: softplus(p) z^2 + z/2; z <= 0: (1/2 + softplus(q)) (e^z - 1 - z) + z/2."""
+
+    def __init__(self, hidden_size: int, intermediate_size: int, activation: str = "xielu", names=("up", "down", "act")):
+        if activation != "xielu":
+            raise ValueError("DenseMLP: activation %r is not implemented" % activation)
+        self.hidden_size, self.intermediate_size, self.names = hidden_size, intermediate_size, names
+        self.w_up = self.w_up_tiled = self.w_down = self.w_down_tiled = self.act = None
+
+    def weight_specs(self, prefix):
+        H, I = self.hidden_size, self.intermediate_size
+        up, down, act = (prefix + "." + n for n in self.names)
+        return [WeightSpec(up, (I, H)), WeightSpec(down, (H, I)), WeightSpec(act, (2,), "bias")]
+
+    def bind(self, prefix, weights):
+        up, down, act = (prefix + "." + n for n in self.names)
+        self.w_up, self.w_up_tiled = ops.weight_forms(weights.pop(up))
+        self.w_down, self.w_down_tiled = ops.weight_forms(weights.pop(down))
+        self.act = weights[act]
+
+    def capturable(self, batch):
+        return True
+
+    def forward(self, x, batch):
+        return ops.linear(ops.linear_xielu(x, self.w_up, self.act, tiled=self.w_up_tiled), self.w_down, tiled=self.w_down_tiled)

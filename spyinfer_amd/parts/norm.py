@@ -11,22 +11,30 @@ from .base import Norm
 
 
 class RMSNorm(Norm):
-    def __init__(self, size: int, eps: float):
+    def __init__(self, size: int, eps: float, suffix: str = ".weight"):
+        """``suffix``: what the weight's name has behind the part's prefix (some checkpoints name the vector by the
+        prefix alone)."""
         self.size = size
         self.eps = float(eps)
+        self.suffix = suffix
         self.weight = None
 
     def weight_specs(self, prefix):
-        return [WeightSpec(prefix + ".weight", (self.size,), "norm")]
+        return [WeightSpec(prefix + self.suffix, (self.size,), "norm")]
 
     def bind(self, prefix, weights):
-        self.weight = weights[prefix + ".weight"]
+        self.weight = weights[prefix + self.suffix]
 
     def capturable(self, batch):
         return True
 
     def add_norm(self, resid, delta, out_dtype, rows=None):
         return ops.add_rms_norm(resid, delta, self.weight, self.eps, out_dtype, rows)
+
+    def add_normed(self, base, y, out=None, copy_dtype=None):
+        """out = base + norm(y) in float32 (the norm on a sublayer's output; ``out`` may be ``base``); returns (out, its
+        copy in ``copy_dtype`` or None)."""
+        return ops.norm_residual(base, y, self.weight, self.eps, out, copy_dtype)
 
     def foldable(self, out_dtype):
         if out_dtype == torch.bfloat16 and self.weight is not None and self.weight.dtype == torch.bfloat16:

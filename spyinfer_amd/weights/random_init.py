@@ -4,7 +4,7 @@ from a configuration and a seed.
 Every tensor is drawn from its own stream keyed by (seed, tensor name), so the
 values do not depend on the order of tensors or on other tensors' shapes:
 matrices ~ N(0, matrix_std), norm scales ~ norm_mean + N(0, norm_std), biases and
-other vectors centred on zero ~ N(0, bias_std), integer tables uniform.  The folder is then read back by name like any other model.
+other vectors centred on zero ~ N(0, bias_std), weights of a mix of n things ~ (1 + N(0, 0.3)) / n, integer tables uniform.  The folder is then read back by name like any other model.
 The reference has no such mode.
 """
 from __future__ import annotations
@@ -20,7 +20,7 @@ from .loader import WeightSpec
 from .safetensors_io import write_file
 
 
-ROLES = ("matrix", "norm", "bias", "table")
+ROLES = ("matrix", "norm", "bias", "table", "mix")
 
 
 def _stream(seed: int, name: str) -> torch.Generator:
@@ -46,6 +46,8 @@ def random_tensors(specs: Iterable[WeightSpec], seed: int, dtype: torch.dtype = 
             out[s.name] = (norm_mean + norm_std * torch.randn(s.shape, generator=g, dtype=torch.float32)).to(dtype)
         elif s.role == "bias":
             out[s.name] = (bias_std * torch.randn(s.shape, generator=g, dtype=torch.float32)).to(dtype)
+        elif s.role == "mix":
+            out[s.name] = ((1.0 + 0.3 * torch.randn(s.shape, generator=g, dtype=torch.float32)) / max(1, s.shape[-1])).to(dtype)
         else:
             # big matrices are filled in row blocks to bound the float32 staging memory
             t = torch.empty(s.shape, dtype=dtype)
@@ -76,6 +78,8 @@ def random_tensors_on_device(specs: Iterable[WeightSpec], seed: int, dtype: torc
             out[s.name] = (norm_mean + norm_std * torch.randn(s.shape, generator=g, dtype=torch.float32, device=device)).to(dtype)
         elif s.role == "bias":
             out[s.name] = (bias_std * torch.randn(s.shape, generator=g, dtype=torch.float32, device=device)).to(dtype)
+        elif s.role == "mix":
+            out[s.name] = ((1.0 + 0.3 * torch.randn(s.shape, generator=g, dtype=torch.float32, device=device)) / max(1, s.shape[-1])).to(dtype)
         else:
             t = torch.empty(s.shape, dtype=dtype, device=device)
             t.normal_(0.0, matrix_std, generator=g)

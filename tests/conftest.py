@@ -21,13 +21,15 @@ def emu_ops(monkeypatch):
     from spyinfer_amd.kernels import ops
     from tests.emu_ops import EmuOps
     emu = EmuOps()
-    for name in ("embedding", "add_rms_norm", "rms_norm", "qk_norm_rope_store", "swiglu", "sample"):
+    for name in ("embedding", "add_rms_norm", "rms_norm", "qk_norm_rope_store", "swiglu", "sample", "pair_embedding", "norm_residual",
+                 "depth_mix", "xielu", "mingru", "gemm_strided", "latent_prepare", "latent_attention"):
         monkeypatch.setattr(ops, name, getattr(emu, name))
 
     def linear(x, w, out_dtype=None, tiled=None, out=None):
         y = emu.linear(x, w, out_dtype)
         return y if out is None else out.copy_(y)
     monkeypatch.setattr(ops, "linear", linear)
+    monkeypatch.setattr(ops, "linear_xielu", lambda x, w, pq, tiled=None: emu.xielu(emu.linear(x, w), pq))
     monkeypatch.setattr(ops, "linear_swiglu", lambda x, w, tiled=None: emu.swiglu(emu.linear(x, w)))
     monkeypatch.setattr(ops, "paged_attention", lambda q, k_cache, v_cache, page_size, meta, n_q, n_kv, d, scale, window, raw=None,
                         for_product=False: emu.paged_attention(q, k_cache, v_cache, page_size, meta, n_q, n_kv, d, scale, window))

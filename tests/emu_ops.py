@@ -99,3 +99,115 @@ class EmuOps:
                 idx = int(torch.searchsorted(c, torch.tensor(float(u[r]), dtype=torch.float64), right=True))
                 out[r] = min(idx, logits.shape[1] - 1)
         return out
+
+    # ---- stream of output-normed layers, kept layer results, recurrences, latent attention ----
+    @staticmethod
+    def _copy(out, copy_dtype):
+        return None if copy_dtype is None or copy_dtype == torch.float32 else out.to(copy_dtype)
+
+    def pair_embedding(self, ids, table, pair, buckets, mul_prev, mul_cur, positions, token_entry, cu_q, slot_ids, last_token,
+                       copy_dtype=None):
+        out = table[ids.long()].float()
+        if pair is not None:
+            old = last_token.clone()
+            for t in range(ids.shape[0]):
+                e = int(token_entry[t])
+                if int(positions[t]) == 0:
+                    row = buckets
+                else:
+                    prev = int(old[int(slot_ids[e])]) if t == int(cu_q[e]) else int(ids[t - 1])
+                    row = (prev * mul_prev + int(ids[t]) * mul_cur) % buckets
+                out[t] += pair[row].float()
+            for e in range(slot_ids.shape[0]):
+                last_token[int(slot_ids[e])] = ids[int(cu_q[e + 1]) - 1]
+        return out, self._copy(out, copy_dtype)
+
+    def norm_residual(self, base, y, weight, eps, out=None, copy_dtype=None):
+        yf = y.float()
+        r = base + yf * torch.rsqrt((yf * yf).mean(-1, keepdim=True) + eps) * weight.float()
+        if out is None:
+            out = r
+        else:
+            out.copy_(r)
+        return out, self._copy(out, copy_dtype)
+
+    def depth_mix(self, kept, n, a, copy_dtype=None):
+        out = torch.zeros_like(kept[0])
+        for j in range(n):
+            out += a[j].float() * kept[j]
+        return out, self._copy(out, copy_dtype)
+
+    def xielu(self, x, pq):
+        sp = torch.nn.functional.softplus
+        z = x.float()
+        ap, aq = sp(pq[0].float()), 0.5 + sp(pq[1].float())
+        x.copy_(torch.where(z > 0, ap * z * z + 0.5 * z, aq * (torch.expm1(torch.clamp(z, max=0)) - z) + 0.5 * z).to(x.dtype))
+        return x
+
+    def mingru(self, zxg, bz, bx, state, pieces, n_pieces, multi, slot_ids):
+        W = zxg.shape[1] // 3
+        f = zxg.float()
+        out = torch.empty((zxg.shape[0], W), dtype=torch.float32)
+        pc = pieces.view(4, n_pieces)
+        for k in range(n_pieces):
+            slot = int(slot_ids[int(pc[0, k])])
+            s = state[slot].clone()
+            for t in range(int(pc[1, k]), int(pc[2, k])):
+                z = torch.sigmoid(f[t, :W] + bz.float())
+                u = f[t, W:2 * W] + bx.float()
+                c = torch.where(u >= 0, u + 0.5, torch.sigmoid(u))
+                s = (1 - z) * s + z * c
+                g = f[t, 2 * W:]
+                out[t] = s * g * torch.sigmoid(g)
+            state[slot] = s            # pieces come in the order of the tokens, so the state walks through them
+        return out.to(zxg.dtype)
+
+    def gemm_strided(self, a, a_strides, b, b_strides, c, c_strides, batch, M, N, K):
+        A = torch.as_strided(a, (batch, M, K), a_strides).float()
+        B = torch.as_strided(b, (batch, N, K), b_strides).float()
+        torch.as_strided(c, (batch, M, N), c_strides).copy_(torch.einsum("bmk,bnk->bmn", A, B).to(c.dtype))
+        return c
+
+    @staticmethod
+    def _rotate(v, p, freq, mag, dims):
+        if not dims:
+            return v
+        half = dims // 2
+        ang = (p.float()[:, None] * freq[None, :].float())
+        c, s = torch.cos(ang) * mag, torch.sin(ang) * mag
+        while c.dim() < v.dim():
+            c, s = c[:, None], s[:, None]
+        a, b = v[..., :half], v[..., half:dims]
+        return torch.cat([a * c - b * s, b * c + a * s, v[..., dims:]], dim=-1)
+
+    def latent_prepare(self, q, dkv, cache, slot_mapping, w_norm, eps, freq, mag, dims, positions, H, DN, DR, R):
+        T = q.shape[0]
+        qa = torch.zeros((T, H, R + DR), dtype=torch.float32)
+        qh = q[:, :H * (DN + DR)].float().reshape(T, H, DN + DR)
+        qa[:, :, R:] = self._rotate(qh[:, :, DN:], positions, freq, mag, dims)
+        if dkv is not None:
+            d = dkv.float()
+            c = d[:, :R] * torch.rsqrt((d[:, :R] ** 2).mean(-1, keepdim=True) + eps) * w_norm.float()
+            rows = torch.cat([c, self._rotate(d[:, R:], positions, freq, mag, dims)], dim=-1).to(cache.dtype)
+            P = cache.shape[1]
+            for t in range(T):
+                sl = int(slot_mapping[t])
+                cache[sl // P, sl % P] = rows[t]
+        return qa
+
+    def latent_attention(self, qa, cache, page_size, meta, sink, R, scale, window, out_dtype):
+        T, H, D = qa.shape
+        out = torch.zeros((T, H, R), dtype=torch.float32)
+        for t in range(T):
+            s, p = int(meta.token_entry[t]), int(meta.positions[t])
+            lo = 0 if not window else max(0, p - window + 1)
+            keys = list(range(lo, p + 1))
+            pages = [int(meta.block_table[s, c // page_size]) for c in keys]
+            assert all(pg >= 0 for pg in pages), "attention reads a page that is not held"
+            rows = cache[pages, [c % page_size for c in keys]].float()
+            sc = (qa[t] @ rows.T) * scale                                  # [H, n]
+            if sink is not None:
+                sc = torch.cat([sc, sink.float()[:, None]], dim=1)
+            pr = torch.softmax(sc, dim=1)[:, :len(keys)]
+            out[t] = pr @ rows[:, :R]
+        return out.to(out_dtype)
