@@ -49,6 +49,109 @@ SHAPES = {
 }
 
 
+def sefevik_shape(width: int, layers: int, vocab: int, window: int = 1024) -> dict:
+    """A Sefevik configuration with the layer sizes of a real model of that width: heads of 128 unrotated and 64 rotated
+    dims, a latent of 512, a feed-forward of three times the width; of every four layers one latent attention with its
+    own rows, two recurrences and one latent attention that reads the first one's rows."""
+    heads = max(1, width // 128)
+    rot = dict(base=10000.0, dims=64, scaling=dict(factor=4.0, original=4096, fast=32.0, slow=1.0))
+    att = dict(heads=heads, dim=128, rot_dim=64, vdim=128, kv_rank=512, scale=192 ** -0.5, mask=dict(size=window), rot=rot)
+    out = []
+    for i in range(layers):
+        kind = i % 4
+        if kind == 0:
+            out.append(dict(type="latent_attention", mixer=dict(att), mlp=dict(kind="dense", ff=3 * width)))
+        elif kind == 3:
+            out.append(dict(type="latent_attention", mixer=dict(att, kv_from=i - 3), mlp=dict(kind="dense", ff=3 * width)))
+        else:
+            out.append(dict(type="mingru", mixer=dict(width=width), mlp=dict(kind="dense", ff=3 * width)))
+    return dict(architecture="Sefevik", vocab=vocab, width=width, norm=dict(eps=1e-5),
+                embedding=dict(bigram=dict(buckets=65521, mul_prev=31, mul_cur=7)), layers=out)
+
+
+def design_compare(args) -> int:
+    """Prefill (one portion of --prefill-tokens) and decode (batch 8 and 32, prompts of --prompt-len) of Sefevik and of
+    Qwen3 at equal width, layers, heads and feed-forward size; ONE JSON line."""
+    import torch
+
+    from spyinfer_amd.config.registry import architecture_of
+    from spyinfer_amd.engine.batch import StepEntry
+    from spyinfer_amd.engine.llm_engine import LLMEngine
+    from spyinfer_amd.engine.runner import bind_weights
+    from spyinfer_amd.kernels import ops
+    from spyinfer_amd.sampling import SamplingParams
+    from spyinfer_amd.weights.random_init import random_tensors_on_device
+
+    ops.hip()
+    dev = torch.device("cuda:0")
+    layers, vocab, page = args.layers or 8, 32768, 16
+    run_dtype = torch.bfloat16 if args.dtype == "bfloat16" else torch.float32
+    g = torch.Generator().manual_seed(args.seed)
+    results = {}
+    for width in [int(x) for x in args.design_sizes.split(",") if x.strip()]:
+        heads = max(1, width // 128)
+        raws = {"sefevik": sefevik_shape(width, layers, vocab),
+                "qwen3": dict(MODEL_8B, num_hidden_layers=layers, hidden_size=width, num_attention_heads=heads,
+                              num_key_value_heads=max(1, heads // 4), intermediate_size=3 * width, vocab_size=vocab)}
+        for name, raw in raws.items():
+            arch = architecture_of(raw)
+            cfg = arch.config_cls.from_dict(raw)
+            model = arch.build(cfg)
+            weights = random_tensors_on_device(model.weight_specs(), args.seed, run_dtype, dev)
+            params = sum(w.numel() for w in weights.values())
+            bind_weights(model, weights, dev, "both")
+            del weights
+            eng = LLMEngine.__new__(LLMEngine)
+            eng._init_with_model(model, dev, dtype=args.dtype, max_model_len=args.context, kvcache_block_size=page,
+                                 num_kvcache_blocks=-(-args.context // page) * 32 + 8, max_num_seqs=32,
+                                 max_num_batched_tokens=max(16384, args.prefill_tokens), enforce_eager=args.enforce_eager, seed=args.seed)
+            out = {"parameters": params}
+            T = args.prefill_tokens
+            best = None
+            for _ in range(4):
+                rc = eng.runner.manager.admit("prefill")
+                eng.runner.manager.reserve(rc, T)
+                toks = torch.randint(0, vocab, (T,), generator=g).tolist()
+                torch.cuda.synchronize()
+                t0 = time.perf_counter()
+                eng.runner.step([StepEntry(rc, toks, [T - 1])])
+                torch.cuda.synchronize()
+                dt = time.perf_counter() - t0
+                eng.runner.manager.release(rc)
+                best = dt if best is None else min(best, dt)
+            out["prefill_%d" % T] = {"tokens_per_s": round(T / best, 1), "ms": round(best * 1e3, 3)}
+            for batch in (8, 32):
+                steps, warm = max(16, args.steps // 4), 8
+                ids = [eng.add_request(torch.randint(0, vocab, (args.prompt_len,), generator=g).tolist(),
+                                       SamplingParams(temperature=0.0, max_new_tokens=steps + warm + 32, ignore_eos=True)) for _ in range(batch)]
+                while any(s.is_prefill or s.num_generated == 0 for s in (eng._sequences[i] for i in ids)):
+                    eng.step()
+                for _ in range(warm):
+                    eng.step()
+                torch.cuda.synchronize()
+                t0 = time.perf_counter()
+                for _ in range(steps):
+                    assert len(eng.step()) == batch
+                torch.cuda.synchronize()
+                dt = time.perf_counter() - t0
+                for i in ids:
+                    eng.remove_request(i)
+                out["decode_b%d" % batch] = {"tokens_per_s": round(batch * steps / dt, 1), "ms_per_step": round(dt / steps * 1e3, 4)}
+            results.setdefault(str(width), {})[name] = out
+            del eng, model
+            torch.cuda.empty_cache()
+    first = results[next(iter(results))]
+    print(json.dumps({
+        "metric": "prefill and decode tok/s of Sefevik beside Qwen3 at equal width, layers, heads and feed-forward size",
+        "value": first["sefevik"]["decode_b8"]["tokens_per_s"], "unit": "tokens/s", "n_gpus": 1, "steps": max(16, args.steps // 4), "warmup": 8,
+        "ms_per_step": first["sefevik"]["decode_b8"]["ms_per_step"], "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "bf16" if args.dtype == "bfloat16" else "fp32", "data": "synthetic (random weights, uniform-random token ids)",
+        "config": {"model": "Sefevik / Qwen3 layer shapes", "layers": layers, "vocab": vocab, "prompt_len": args.prompt_len,
+                   "prefill_tokens": args.prefill_tokens, "window": 1024, "graphs": not args.enforce_eager, "parallelism": "single GPU"},
+        "widths": results}))
+    return 0
+
+
 def main() -> int:
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -75,7 +178,13 @@ def main() -> int:
     ap.add_argument("--serve", type=int, default=0, metavar="N",
                     help="instead of the decode steps: N requests arriving at once, prompts of 128..2048 and outputs of 64..512 "
                          "tokens (uniform), run until all have ended; the value is generated tokens per second of the whole run")
+    ap.add_argument("--design", default="", choices=["", "sefevik"],
+                    help="instead of the decode steps: prefill and decode throughput of that design at a few layer sizes "
+                         "beside the Qwen3 shape of equal width, layers, heads and feed-forward size (--design-sizes)")
+    ap.add_argument("--design-sizes", default="1024,2048,4096", help="widths for --design")
     args = ap.parse_args()
+    if args.design:
+        return design_compare(args)
     if args.gpus != 1:
         print("bench.py: this engine runs on one GPU; --gpus %d is not supported" % args.gpus)
         return 2

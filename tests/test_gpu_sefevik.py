@@ -1,0 +1,222 @@
+"""Sefevik on the GPU: every mechanism's kernel against the plain implementation's function, then whole models through
+the trace replay (the engine's step function, cache manager and kernels) under every schedule, long decoding, and
+greedy generation through the entry point with and without captured steps."""
+import os
+import subprocess
+import sys
+
+import pytest
+import torch
+
+from tests import replay_cases as rc
+from tests import sefevik_cases as sc
+from tests.gpu_util import close, require_gpu
+from tests.plain import sefevik_plain as plain
+
+pytestmark = pytest.mark.gpu
+TOL = {"float32": dict(atol=2e-4, rtol=2e-4), "bfloat16": dict(atol=1e-1, rtol=3e-2)}
+DT = {"float32": torch.float32, "bfloat16": torch.bfloat16}
+
+
+def i32(values, dev):
+    return torch.tensor(values, dtype=torch.int32, device=dev)
+
+
+# ---- mechanisms --------------------------------------------------------------------------------
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_pair_embedding_keeps_the_previous_token_in_the_slot(dtype):
+    from spyinfer_amd.kernels import ops
+    dev = require_gpu()
+    g = torch.Generator().manual_seed(1)
+    V, H, buckets, mp, mc = 37, 24, 11, 5, 3
+    table = torch.randn((V, H), generator=g).to(DT[dtype])
+    pair = torch.randn((buckets + 1, H), generator=g).to(DT[dtype])
+    seqs = {2: torch.randint(0, V, (9,), generator=g).tolist(), 0: torch.randint(0, V, (4,), generator=g).tolist()}
+    last = torch.full((3,), -7, dtype=torch.int32, device=dev)
+    got = {s: [] for s in seqs}
+    # step 1: 5 tokens of slot 2 and 1 of slot 0; step 2: the rest (the entries' first tokens read the slots)
+    for cuts in ({2: (0, 5), 0: (0, 1)}, {0: (1, 4), 2: (5, 9)}):
+        ids, pos, ent, cu, slots = [], [], [], [0], []
+        for e, (s, (lo, hi)) in enumerate(cuts.items()):
+            ids += seqs[s][lo:hi]; pos += list(range(lo, hi)); ent += [e] * (hi - lo); cu.append(len(ids)); slots.append(s)
+        out, copy = ops.pair_embedding(i32(ids, dev), table.to(dev), pair.to(dev), buckets, mp, mc, i32(pos, dev), i32(ent, dev),
+                                       i32(cu, dev), i32(slots, dev), last, DT[dtype])
+        assert (copy is None) == (dtype == "float32")
+        for e, s in enumerate(cuts):
+            got[s].append(out[cu[e]:cu[e + 1]].cpu())
+    for s, toks in seqs.items():
+        rows = plain.bigram_rows(toks, buckets, mp, mc)
+        ref = table.double()[toks] + pair.double()[rows]
+        close(torch.cat(got[s]), ref, torch.float32, what="pair embedding, slot %d" % s)
+    assert last.tolist() == [seqs[0][-1], -7, seqs[2][-1]]
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_stream_kernels(dtype):
+    from spyinfer_amd.kernels import ops
+    dev = require_gpu()
+    g = torch.Generator().manual_seed(2)
+    T, H, eps = 13, 50, 1e-5
+    base, y = torch.randn((T, H), generator=g), (3 * torch.randn((T, H), generator=g)).to(DT[dtype])
+    w = (1 + 0.2 * torch.randn((H,), generator=g)).to(DT[dtype])
+    out, copy = ops.norm_residual(base.to(dev), y.to(dev), w.to(dev), eps, None, DT[dtype])
+    ref = base.double() + plain.rms_norm(y.double(), w.double(), eps)
+    close(out, ref, torch.float32, what="norm_residual")
+    if copy is not None:
+        close(copy, ref, torch.bfloat16, what="norm_residual copy")
+    kept = torch.randn((6, T, H), generator=g)
+    a = torch.randn((4,), generator=g).to(DT[dtype])
+    out, _ = ops.depth_mix(kept.to(dev), 4, a.to(dev), DT[dtype])
+    close(out, sum(a[j].double() * kept[j].double() for j in range(4)), torch.float32, what="depth_mix")
+    z = (2 * torch.randn((T, H), generator=g)).to(DT[dtype])
+    for pq in ((0.3, -0.4), (-2.0, 1.5)):
+        t = torch.tensor(pq).to(DT[dtype])
+        got = ops.xielu(z.clone().to(dev), t.to(dev))
+        close(got, plain.xielu(z.double(), float(t[0]), float(t[1])), DT[dtype], what="xielu %r" % (pq,))
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_mingru_scan_in_pieces_carries_the_state(dtype):
+    from spyinfer_amd.engine.batch import StepBatch  # noqa: F401  (the pieces are planned as the part plans them)
+    from spyinfer_amd.kernels import ops
+    from spyinfer_amd.parts import recurrent
+    dev = require_gpu()
+    g = torch.Generator().manual_seed(3)
+    W, lens = 70, [150, 1, 33]
+    zxg = torch.randn((sum(lens) * 2, 3 * W), generator=g).to(DT[dtype])
+    bz, bx = torch.randn((W,), generator=g).to(DT[dtype]), torch.randn((W,), generator=g).to(DT[dtype])
+    state = torch.zeros((5, W), dtype=torch.float32, device=dev)
+    slots = [3, 0, 4]
+
+    class FakeBatch:
+        def __init__(self, ls):
+            import numpy as np
+            self.S, self.lens, self.shared, self.arrays = len(ls), np.asarray(ls, dtype=np.int32), {}, {}
+            self._cu = np.concatenate([[0], np.cumsum(ls)]).astype(np.int32)
+
+        def host_array(self, name):
+            return self._cu
+
+        def add_array(self, name, values):
+            self.arrays[name] = values
+    outs, row = [[] for _ in lens], 0
+    for step in range(2):                                   # two steps: the second starts from the first's state
+        fb = FakeBatch(lens)
+        recurrent.plan_scan_pieces(fb)
+        n, multi = fb.shared["scan_pieces"]
+        assert multi and n == sum(-(-l // recurrent.SCAN_PIECE) for l in lens)
+        x = zxg[row:row + sum(lens)]
+        y = ops.mingru(x.to(dev), bz.to(dev), bx.to(dev), state, i32(fb.arrays["scan_pieces"], dev), n, multi, i32(slots, dev))
+        at = 0
+        for e, l in enumerate(lens):
+            outs[e].append((x[at:at + l], y[at:at + l].cpu()))
+            at += l
+        row += sum(lens)
+    for e in range(len(lens)):
+        x = torch.cat([a for a, _ in outs[e]]).double()
+        z = torch.sigmoid(x[:, :W] + bz.double())
+        u = x[:, W:2 * W] + bx.double()
+        c = torch.where(u >= 0, u + 0.5, torch.sigmoid(u))
+        s, ref = torch.zeros(W, dtype=torch.float64), []
+        for t in range(x.shape[0]):
+            s = (1 - z[t]) * s + z[t] * c[t]
+            ref.append(s * x[t, 2 * W:] * torch.sigmoid(x[t, 2 * W:]))
+        close(torch.cat([b for _, b in outs[e]]), torch.stack(ref), DT[dtype], what="mingru entry %d" % e)
+        close(state[slots[e]], s, torch.float32, what="mingru state %d" % e)
+
+
+# ---- whole models under every schedule ------------------------------------------------------------
+MODELS = {"a": (sc.SEF_A, 3, None), "b": (sc.SEF_B, 4, None), "c": (sc.SEF_C, 6, None), "a_sharp": (sc.SEF_A, 5, sc.sharpen()),
+          "far_sharp": (sc.SEF_FAR, 8, sc.sharpen(8.0))}
+
+
+@pytest.fixture(scope="module")
+def folders(tmp_path_factory):
+    return {name: sc.write_model(str(tmp_path_factory.mktemp("gsef_" + name)), cfg, seed, tweak) for name, (cfg, seed, tweak) in MODELS.items()}
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("name", ["a", "b", "c", "a_sharp"])
+@pytest.mark.parametrize("mode", ["whole", "bulk_tail", "portions", "mixed"])
+def test_schedules_equal_the_plain_implementation(folders, name, mode, dtype, tmp_path):
+    require_gpu()
+    folder = folders[name]
+    requests = rc.random_requests(sc.vocab_of(folder), [41, 1, 2, 130, 23, 30, 52, 38, 75], 7)
+    steps = {"whole": rc.whole, "bulk_tail": lambda r: rc.bulk_tail(r, 40), "portions": rc.portions, "mixed": rc.mixed}[mode](requests)
+    rc.run_replay_inprocess(folder, dtype, str(tmp_path), steps, rc.max_live_tokens(steps),
+                            ["--kvcache-block-size", "8" if name != "c" else "16", "--poison-cache"])
+    rc.compare(rc.collect(str(tmp_path), steps, sc.vocab_of(folder)), sc.plain_logits(folder, requests),
+               what="%s/%s/%s" % (name, mode, dtype), **TOL[dtype])
+
+
+@pytest.mark.parametrize("mode", ["whole", "bulk_tail", "portions"])
+def test_far_keys_among_hundreds(folders, mode, tmp_path):
+    """One attention layer without a window and with sharp scores: the keys that decide a row's result lie anywhere in
+    600 tokens, across many pages."""
+    require_gpu()
+    folder = folders["far_sharp"]
+    requests = rc.random_requests(sc.vocab_of(folder), [600, 333], 12)
+    steps = {"whole": rc.whole, "bulk_tail": lambda r: rc.bulk_tail(r, 50), "portions": lambda r: rc.portions(r, (100, 3, 2, 257, 64, 1))}[mode](requests)
+    rc.run_replay_inprocess(folder, "float32", str(tmp_path), steps, rc.max_live_tokens(steps), ["--poison-cache"])
+    rc.compare(rc.collect(str(tmp_path), steps, sc.vocab_of(folder)), sc.plain_logits(folder, requests), what="far/" + mode, **TOL["float32"])
+
+
+def test_long_decoding_passes_many_windows(folders, tmp_path):
+    require_gpu()
+    folder = folders["a"]
+    requests = rc.random_requests(97, [260], 13)
+    steps = rc.bulk_tail(requests, 250)
+    rc.run_replay_inprocess(folder, "float32", str(tmp_path), steps, rc.max_live_tokens(steps), ["--kvcache-block-size", "8", "--poison-cache"])
+    rc.compare(rc.collect(str(tmp_path), steps, 97), sc.plain_logits(folder, requests), what="long decoding", **TOL["float32"])
+
+
+# ---- the entry point ---------------------------------------------------------------------------
+@pytest.mark.parametrize("eager", [True, False])
+def test_greedy_generation_equals_plain(folders, eager):
+    from spyinfer_amd.engine.llm_engine import LLMEngine
+    from spyinfer_amd.sampling import SamplingParams
+    require_gpu()
+    folder = folders["a"]
+    model = plain.PlainSefevik.from_folder(folder)
+    prompts = list(rc.random_requests(97, [5, 17, 2, 30, 9], 9).values())
+    want = [model.greedy(p, 24) for p in prompts]
+    for opts in (dict(), dict(max_num_batched_tokens=12, prefill_chunk=7, max_num_seqs=2)):
+        kw = dict(dtype="float32", max_model_len=64, num_kvcache_blocks=24, max_num_seqs=4, kvcache_block_size=8, enforce_eager=eager)
+        kw.update(opts)
+        eng = LLMEngine(folder, **kw)
+        assert eng.generate(prompts, SamplingParams(max_new_tokens=24, ignore_eos=True)) == want
+        if not eager:
+            assert eng.runner.graph_replays > 0
+        eng.runner.manager.check()
+
+
+def test_bfloat16_generation_follows_the_plain_logits(folders):
+    from spyinfer_amd.engine.llm_engine import LLMEngine
+    from spyinfer_amd.sampling import SamplingParams
+    require_gpu()
+    folder = folders["c"]
+    model = plain.PlainSefevik.from_folder(folder)
+    prompts = list(rc.random_requests(400, [33, 70, 8], 10).values())
+    eng = LLMEngine(folder, dtype="bfloat16", max_model_len=128, num_kvcache_blocks=40, max_num_seqs=4)
+    outs = eng.generate(prompts, SamplingParams(max_new_tokens=12, ignore_eos=True))
+    for p, out in zip(prompts, outs):
+        toks = list(p)
+        for t in out:
+            logits = model.forward(toks)[-1]
+            best = int(torch.argmax(logits))
+            assert t == best or float(logits[best] - logits[t]) < 0.15, "token %d where the plain logits prefer %d clearly" % (t, best)
+            toks.append(t)
+
+
+def test_trace_run_as_a_program(folders, tmp_path):
+    require_gpu()
+    folder = folders["b"]
+    requests = rc.random_requests(61, [19, 40], 14)
+    steps = rc.portions(requests)
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    import json
+    r = subprocess.run([sys.executable, os.path.join(root, "bin", "trace_run"), "--model", folder, "--dtype", "float32", "--out", str(tmp_path),
+                        "--max-tokens", str(rc.max_live_tokens(steps))], input="".join(json.dumps(s) + "\n" for s in steps),
+                       capture_output=True, text=True, timeout=600)
+    assert r.returncode == 0, r.stderr[-2000:]
+    rc.compare(rc.collect(str(tmp_path), steps, 61), sc.plain_logits(folder, requests), what="trace_run", **TOL["float32"])
