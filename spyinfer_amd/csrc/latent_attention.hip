@@ -224,3 +224,246 @@ extern "C" int spy_latent_attention(void* out, int out_dtype, const float* qa, c
     SPY_CHECK_LAUNCH("spy_latent_attention");
     return 0;
 }
+
+// ---------------------------------------------------------------------------------------------
+// The same attention on MFMA for bfloat16 caches.  All heads of a token read the same latent rows, so the query rows of
+// an entry, (token, head) pairs, token major, are one long list against one "kv head": a block of LW waves takes
+// 16 LW consecutive rows (a row tile per wave), walks the keys that its rows' tokens see in chunks of 32, and stages every
+// chunk in LDS ONCE for all its waves, in two forms: rows [key][D] for S^T = K . Q^T and, for the first R values, the
+// transpose [d][key] for O^T += V^T . P^T (the values are the keys' first part: no second read of memory).  With
+// v_mfma_f32_16x16x32_bf16 tile a of S^T takes keys 8 (r / 4) + r % 4 and tile b those + 4, so that lane (q row, g) holds
+// the scores of keys 8 g .. 8 g + 7, exactly the 8 k values of its P^T operand.  Softmax float32, online, the sink in
+// the first part's start (m = sink, l = 1).  grid.y parts of the keys (steps of single tokens): the parts' (O, m, l) go
+// to a workspace and a second kernel adds them.
+typedef __attribute__((__vector_size__(8 * sizeof(short)))) short lbf16x8_t;
+typedef __attribute__((__vector_size__(4 * sizeof(float)))) float lf32x4_t;
+typedef __attribute__((__vector_size__(4 * sizeof(uint32_t)))) uint32_t lu32x4_t;
+
+#define LW 4          // waves (row tiles) per block
+#define LKPAD 8       // bf16 of padding per staged key row
+#define LVROW 40      // bf16 per row of the transposed values (32 keys + 8 of padding)
+
+// QS: most 32-wide steps of D; RT: most 16-wide tiles of R (both bound the registers)
+template <int QS, int RT, typename TW>
+__global__ __launch_bounds__(LW * 64) void latent_attention_mfma_kernel(
+    bf16_t* __restrict__ out, float* __restrict__ ws, const float* __restrict__ qa, const bf16_t* __restrict__ cache, int P,
+    int num_pages, const int* __restrict__ cu_q, const int* __restrict__ pos0, const int* __restrict__ kv_len,
+    const int* __restrict__ block_table, int max_blocks, const int* __restrict__ tile_entry, const int* __restrict__ tile_row0,
+    const TW* __restrict__ sink, int H, int R, int D, float scale, int window) {
+    extern __shared__ __attribute__((aligned(16))) unsigned char lds_raw[];
+    const int tid = threadIdx.x, wave = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63, r16 = lane & 15, g = lane >> 4;
+    const int tile = blockIdx.x, sp = blockIdx.y, splits = gridDim.y;
+    const int e = tile_entry[tile];
+    if (e < 0) return;
+    const int q0 = cu_q[e];
+    const int n_rows = (cu_q[e + 1] - q0) * H;
+    const int r_lo = tile_row0[tile];
+    if (r_lo >= n_rows) return;
+    const int r_hi = min(r_lo + 16 * LW, n_rows) - 1;
+    const int p0 = pos0[e], kvl = kv_len[e];
+    const int p_lo = p0 + r_lo / H, p_hi = min(p0 + r_hi / H, kvl - 1);
+    const int lo = window > 0 ? max(0, p_lo - window + 1) : 0;
+    const int c_start = lo & ~31;
+    const int n_chunks = (p_hi - c_start) / 32 + 1;
+    const int c_begin = (int)((long long)n_chunks * sp / splits), c_end = (int)((long long)n_chunks * (sp + 1) / splits);
+    const int q_steps = (D + 31) / 32, r_tiles = (R + 15) / 16;
+    const int Dp = q_steps * 32, krow = Dp + LKPAD;
+    bf16_t* Ks = reinterpret_cast<bf16_t*>(lds_raw);                  // [32][krow]
+    bf16_t* Vt = Ks + 32 * krow;                                       // [r_tiles * 16][LVROW]
+    // this lane's query row
+    const int row = r_lo + 16 * wave + r16;
+    const bool row_ok = row <= r_hi;
+    const int prow = p0 + row / H, head = row % H;
+    const int lo_row = window > 0 ? prow - window + 1 : 0;
+    lbf16x8_t bq[QS];
+    {
+        const float* qv = qa + ((size_t)q0 * H + row) * D;
+#pragma unroll
+        for (int s = 0; s < QS; ++s) {
+            const int d0 = 32 * s + 8 * g;
+            lu32x4_t packed = {0u, 0u, 0u, 0u};
+            if (s < q_steps && row_ok && d0 < D) {
+                const float4 x = *reinterpret_cast<const float4*>(qv + d0), y = *reinterpret_cast<const float4*>(qv + d0 + 4);
+                packed = lu32x4_t{pack_bf16x2(x.x, x.y), pack_bf16x2(x.z, x.w), pack_bf16x2(y.x, y.y), pack_bf16x2(y.z, y.w)};
+            }
+            bq[s] = __builtin_bit_cast(lbf16x8_t, packed);
+        }
+    }
+    const bool with_sink = sink != nullptr && sp == 0;
+    float m = with_sink && row_ok ? to_f32<TW>(sink[head]) : -INFINITY;
+    float l = with_sink && row_ok && g == 0 ? 1.f : 0.f;          // a row's sum is spread over its four lanes
+    lf32x4_t acc[RT];
+#pragma unroll
+    for (int i = 0; i < RT; ++i) acc[i] = lf32x4_t{0.f, 0.f, 0.f, 0.f};
+    const int* bt = block_table + (size_t)e * max_blocks;
+    const int pieces_per_key = Dp / 8, pieces = 32 * pieces_per_key;
+    const int ka_row = 8 * (r16 >> 2) + (r16 & 3);                  // tile a's key of this lane's operand row; tile b: + 4
+    for (int c = c_begin; c < c_end; ++c) {
+        const int key0 = c_start + 32 * c;
+        __syncthreads();                                             // the chunk before is read
+        for (int i = tid; i < pieces; i += LW * 64) {
+            const int k = i / pieces_per_key, d8 = (i - k * pieces_per_key) * 8;
+            const int key = key0 + k;
+            lu32x4_t v = {0u, 0u, 0u, 0u};
+            if (key >= lo && key <= p_hi && d8 < D) {
+                const int page = bt[key / P];
+                if (page >= 0 && page < num_pages) v = *reinterpret_cast<const lu32x4_t*>(cache + ((size_t)page * P + key % P) * D + d8);
+            }
+            *reinterpret_cast<lu32x4_t*>(Ks + k * krow + d8) = v;
+            if (d8 < r_tiles * 16) {
+#pragma unroll
+                for (int j = 0; j < 4; ++j) {
+                    Vt[(d8 + 2 * j) * LVROW + k] = (bf16_t)(v[j] & 0xffffu);
+                    Vt[(d8 + 2 * j + 1) * LVROW + k] = (bf16_t)(v[j] >> 16);
+                }
+            }
+        }
+        __syncthreads();
+        // ---- S^T = K . Q^T ----
+        lf32x4_t sa = {0.f, 0.f, 0.f, 0.f}, sb = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int s = 0; s < QS; ++s) {
+            if (s < q_steps) {
+                const lbf16x8_t ka = *reinterpret_cast<const lbf16x8_t*>(Ks + ka_row * krow + 32 * s + 8 * g);
+                const lbf16x8_t kb = *reinterpret_cast<const lbf16x8_t*>(Ks + (ka_row + 4) * krow + 32 * s + 8 * g);
+                sa = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ka, bq[s], sa, 0, 0, 0);
+                sb = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kb, bq[s], sb, 0, 0, 0);
+            }
+        }
+        // ---- softmax over this lane's 8 keys of its row ----
+        float sc[8];
+        float bmax = -INFINITY;
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+            const int key = key0 + 8 * g + j;
+            const float v = (j < 4 ? sa[j] : sb[j - 4]) * scale;
+            const bool ok = row_ok && key <= prow && key >= lo_row && key < kvl;
+            sc[j] = ok ? v : -INFINITY;
+            bmax = fmaxf(bmax, sc[j]);
+        }
+        bmax = fmaxf(bmax, __shfl_xor(bmax, 16, 64));
+        bmax = fmaxf(bmax, __shfl_xor(bmax, 32, 64));
+        const float m_new = fmaxf(m, bmax);
+        float alpha = 1.f;
+        lbf16x8_t pb = {0, 0, 0, 0, 0, 0, 0, 0};
+        if (m_new != -INFINITY) {
+            alpha = (m == -INFINITY) ? 0.f : __expf(m - m_new);
+            float psum = 0.f;
+#pragma unroll
+            for (int j = 0; j < 8; ++j) {
+                const float pj = (sc[j] == -INFINITY) ? 0.f : __expf(sc[j] - m_new);
+                psum += pj;
+                pb[j] = (short)f32_to_bf16(pj);
+            }
+            l = l * alpha + psum;
+            m = m_new;
+        }
+        // ---- O^T = O^T * alpha + V^T . P^T ----
+#pragma unroll
+        for (int i = 0; i < RT; ++i) {
+            if (i < r_tiles) {
+                const lbf16x8_t vt = *reinterpret_cast<const lbf16x8_t*>(Vt + (16 * i + r16) * LVROW + 8 * g);
+                acc[i] *= alpha;
+                acc[i] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vt, pb, acc[i], 0, 0, 0);
+            }
+        }
+    }
+    // the row's sum over its four lanes
+    l += __shfl_xor(l, 16, 64);
+    l += __shfl_xor(l, 32, 64);
+    if (!row_ok) return;
+    // lane (row r16, g) holds O^T[v = 16 i + 4 g + j][row], j < 4
+    if (splits == 1) {
+        const float inv = l > 0.f ? 1.0f / l : 0.f;
+        bf16_t* o = out + ((size_t)q0 * H + row) * R;
+#pragma unroll
+        for (int i = 0; i < RT; ++i) {
+            const int v0 = 16 * i + 4 * g;
+            if (i < r_tiles && v0 < R) {               // R % 4 == 0 (checked by the launcher)
+                uint2 w;
+                w.x = pack_bf16x2(acc[i][0] * inv, acc[i][1] * inv);
+                w.y = pack_bf16x2(acc[i][2] * inv, acc[i][3] * inv);
+                *reinterpret_cast<uint2*>(o + v0) = w;
+            }
+        }
+        return;
+    }
+    // parts: ws[(global row * splits + part)] = { O[R] unnormalised, m, l }
+    float* w = ws + (((size_t)q0 * H + row) * splits + sp) * (R + 2);
+#pragma unroll
+    for (int i = 0; i < RT; ++i) {
+        const int v0 = 16 * i + 4 * g;
+        if (i < r_tiles && v0 < R) {
+#pragma unroll
+            for (int j = 0; j < 4; ++j) w[v0 + j] = acc[i][j];
+        }
+    }
+    if (g == 0) { w[R] = m; w[R + 1] = l; }
+}
+
+// out[row] = sum_i O_i e^(m_i - M) / sum_i l_i e^(m_i - M) over the parts i of a row, added in ascending i
+__global__ __launch_bounds__(256) void latent_attention_merge_kernel(bf16_t* __restrict__ out, const float* __restrict__ ws, int R, int splits) {
+    __shared__ float wgt[64];
+    __shared__ float inv_l;
+    const size_t row = blockIdx.x;
+    const float* base = ws + row * splits * (R + 2);
+    if (threadIdx.x == 0) {
+        float M = -INFINITY;
+        for (int i = 0; i < splits; ++i) M = fmaxf(M, base[(size_t)i * (R + 2) + R]);
+        float L = 0.f;
+        for (int i = 0; i < splits; ++i) {
+            const float mi = base[(size_t)i * (R + 2) + R];
+            const float e = (mi == -INFINITY) ? 0.f : expf(mi - M);
+            wgt[i] = e;
+            L += base[(size_t)i * (R + 2) + R + 1] * e;
+        }
+        inv_l = L > 0.f ? 1.0f / L : 0.f;
+    }
+    __syncthreads();
+    for (int j = threadIdx.x; j < R; j += blockDim.x) {
+        float o = 0.f;
+        for (int i = 0; i < splits; ++i) o = fmaf(base[(size_t)i * (R + 2) + j], wgt[i], o);
+        out[row * R + j] = f32_to_bf16(o * inv_l);
+    }
+}
+
+extern "C" long long spy_latent_attention_mfma_workspace(int T, int H, int R, int splits) {
+    return splits > 1 ? (long long)T * H * splits * (R + 2) : 0;
+}
+
+// tiles: num_tiles records (entry, first row) of 64 rows each.  ws: float32, spy_latent_attention_mfma_workspace values.
+extern "C" int spy_latent_attention_mfma(void* out, float* ws, const float* qa, const void* cache, int P, int num_pages,
+                                         const int* cu_q, const int* pos0, const int* kv_len, const int* block_table,
+                                         int max_blocks, const int* tile_entry, const int* tile_row0, int num_tiles,
+                                         const void* sink, int sink_dtype, int T, int H, int R, int DR, float scale, int window,
+                                         int splits, hipStream_t st) {
+    const int D = R + DR;
+    SPY_REQUIRE(T > 0 && H > 0 && R > 0 && DR >= 0 && P > 0 && num_pages > 0 && max_blocks > 0 && num_tiles > 0,
+                "spy_latent_attention_mfma: empty operand");
+    SPY_REQUIRE(D % 8 == 0 && R % 8 == 0 && D <= 640 && R <= 512, "spy_latent_attention_mfma: rows of %d + %d values are not taken", R, DR);
+    SPY_REQUIRE(splits >= 1 && splits <= 64 && (splits == 1 || ws), "spy_latent_attention_mfma: %d parts (1..64, with a workspace)", splits);
+    SPY_REQUIRE(((uintptr_t)qa % 16) == 0 && ((uintptr_t)cache % 16) == 0 && ((uintptr_t)out % 8) == 0, "spy_latent_attention_mfma: operands are not aligned");
+    const int q_steps = (D + 31) / 32, r_tiles = (R + 15) / 16;
+    const size_t lds = ((size_t)32 * (q_steps * 32 + LKPAD) + (size_t)r_tiles * 16 * LVROW) * sizeof(bf16_t);
+    const dim3 grid(num_tiles, splits);
+#define SPY_LA_LAUNCH(QS, RT)                                                                                                   \
+    SPY_DISPATCH(sink_dtype, TW, {                                                                                              \
+        auto kernel = latent_attention_mfma_kernel<QS, RT, TW>;                                                                 \
+        if (lds > 48 * 1024) {                                                                                                  \
+            hipError_t e_ = hipFuncSetAttribute((const void*)kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);      \
+            if (e_ != hipSuccess) return spy_fail("spy_latent_attention_mfma: %zu bytes of LDS refused: %s", lds, hipGetErrorString(e_)); \
+        }                                                                                                                       \
+        kernel<<<grid, LW * 64, lds, st>>>((bf16_t*)out, ws, qa, (const bf16_t*)cache, P, num_pages, cu_q, pos0, kv_len,        \
+                                           block_table, max_blocks, tile_entry, tile_row0, (const TW*)sink, H, R, D, scale, window); \
+    })
+    if (q_steps <= 8 && r_tiles <= 8) { SPY_LA_LAUNCH(8, 8); }
+    else if (q_steps <= 12 && r_tiles <= 16) { SPY_LA_LAUNCH(12, 16); }
+    else { SPY_LA_LAUNCH(20, 32); }
+#undef SPY_LA_LAUNCH
+    SPY_CHECK_LAUNCH("spy_latent_attention_mfma");
+    if (splits > 1) {
+        latent_attention_merge_kernel<<<(unsigned)((size_t)T * H), R >= 256 ? 256 : 64, 0, st>>>((bf16_t*)out, ws, R, splits);
+        SPY_CHECK_LAUNCH("spy_latent_attention_mfma (merge)");
+    }
+    return 0;
+}

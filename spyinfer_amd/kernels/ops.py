@@ -76,7 +76,7 @@ class _Hip:
                      "spy_sample", "spy_sample_workspace", "spy_gemm_skinny", "spy_gemm_skinny_swiglu",
                      "spy_gemm_decode", "spy_gemm_decode_workspace", "spy_embedding_sumsq", "spy_sample_static", "spy_measure_read",
                      "spy_pair_embedding", "spy_norm_residual", "spy_depth_mix", "spy_xielu", "spy_mingru", "spy_latent_prepare",
-                     "spy_gemm_strided", "spy_latent_attention"):
+                     "spy_gemm_strided", "spy_latent_attention", "spy_latent_attention_mfma", "spy_latent_attention_mfma_workspace"):
             if not hasattr(self.lib, name):
                 raise KernelError("the kernel library %s lacks %s: it is older than its sources; build it again "
                                   "(spyinfer_amd.kernels.build.build())" % (self.lib._name, name))
@@ -1010,8 +1010,24 @@ def latent_prepare(q: torch.Tensor, dkv: Optional[torch.Tensor], cache: Optional
     return qa
 
 
+LATENT_TILE_ROWS = 64       # query rows, (token, head) pairs, of one block of the MFMA latent attention
+LATENT_MFMA = True          # False forces the plain kernel for bfloat16 too (tests flip it; nothing else does)
+
+
+def latent_attention_mfma_ok(dtype, R: int, D: int) -> bool:
+    """Whether the MFMA kernel takes latent rows of D values of which R are the values: bfloat16, 16-byte pieces, and
+    sums of a row tile that fit a wave's registers."""
+    return LATENT_MFMA and dtype == torch.bfloat16 and D % 8 == 0 and R % 8 == 0 and D <= 640 and R <= 512
+
+
+def latent_key_parts(num_tiles: int, max_keys: int) -> int:
+    """Parts into which the MFMA latent attention cuts every tile's keys so that a step of few tiles (single tokens)
+    still has blocks for the whole device; a part wants 64 keys at least."""
+    return max(1, min(512 // max(1, num_tiles), 16, -(-max_keys // 64)))
+
+
 def latent_attention(qa: torch.Tensor, cache: torch.Tensor, page_size: int, meta: "AttentionMeta", sink: Optional[torch.Tensor],
-                     R: int, scale: float, window: Optional[int], out_dtype: torch.dtype) -> torch.Tensor:
+                     R: int, scale: float, window: Optional[int], out_dtype: torch.dtype, tiles=None, key_parts: int = 1) -> torch.Tensor:
     """Attention of ``qa [T, H, R + DR]`` (float32, absorbed queries) over the latent rows ``cache [pages, P, R + DR]``:
     score = qa . row * scale, softmax with exp(sink[h]) added to the denominator, causal with ``window``; the result is
     sum_j p_j row_j[:R], [T, H, R] in ``out_dtype``."""
@@ -1023,6 +1039,21 @@ def latent_attention(qa: torch.Tensor, cache: torch.Tensor, page_size: int, meta
     _check(sink is None or sink.shape == (H,), "latent_attention: one sink per head expected")
     _check(meta.block_table.shape == (meta.S, meta.max_blocks), "latent_attention: block table must be [S, max_blocks]")
     out = torch.empty((T, H, R), dtype=out_dtype, device=qa.device)
+    if T and tiles is not None and out_dtype == torch.bfloat16 and latent_attention_mfma_ok(cache.dtype, R, D):
+        # tiles: (entry [n], first row [n], n) of LATENT_TILE_ROWS rows each, planned on the host
+        tile_entry, tile_row0, n = tiles
+        _dev(tile_entry, tile_row0, meta.cu_q, meta.pos0)
+        _check(n > 0 and tile_entry.shape == (n,) and tile_row0.shape == (n,), "latent_attention: the tiles' arrays do not fit their number")
+        ws = None
+        if key_parts > 1:
+            ws = torch.empty((hip().lib.spy_latent_attention_mfma_workspace(ctypes.c_int(T), ctypes.c_int(H), ctypes.c_int(R),
+                                                                            ctypes.c_int(key_parts)),), dtype=torch.float32, device=qa.device)
+        hip().call("spy_latent_attention_mfma", _ptr(out), _ptr(ws), _ptr(qa), _ptr(cache), ctypes.c_int(page_size),
+                   ctypes.c_int(cache.shape[0]), _ptr(meta.cu_q), _ptr(meta.pos0), _ptr(meta.kv_len), _ptr(meta.block_table),
+                   ctypes.c_int(meta.max_blocks), _ptr(tile_entry), _ptr(tile_row0), ctypes.c_int(n), _ptr(sink),
+                   _code(sink, "sink") if sink is not None else F32, ctypes.c_int(T), ctypes.c_int(H), ctypes.c_int(R),
+                   ctypes.c_int(D - R), ctypes.c_float(scale), ctypes.c_int(int(window or 0)), ctypes.c_int(key_parts), _Hip.stream())
+        return out
     if T:
         hip().call("spy_latent_attention", _ptr(out), _code(out, "out"), _ptr(qa), _ptr(cache), _code(cache, "cache"),
                    ctypes.c_int(page_size), ctypes.c_int(cache.shape[0]), _ptr(meta.kv_len), _ptr(meta.block_table),

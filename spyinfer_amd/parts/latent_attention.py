@@ -14,6 +14,7 @@ from __future__ import annotations
 
 from typing import Optional
 
+import numpy as np
 import torch
 
 from ..cache.spec import PagedRows
@@ -83,6 +84,32 @@ class LatentAttention(Mixer):
     def capturable(self, batch):
         return True
 
+    def plan(self, batch) -> None:
+        """The step's query rows, (token, head) pairs of each entry, cut into tiles for the MFMA kernel, and the number
+        of parts of a tile's keys (a launch shape: it goes into a captured step's key)."""
+        if not ops.latent_attention_mfma_ok(batch.act_dtype, self.kv_rank, self.kv_rank + self.rot_dim):
+            return
+        note = ("latent_tiles", self.heads)
+        if note not in batch.shared:
+            rows = batch.lens.astype(np.int64) * self.heads
+            size = ops.LATENT_TILE_ROWS
+            counts = (rows + size - 1) // size
+            entry = np.repeat(np.arange(batch.S, dtype=np.int64), counts)
+            first = np.zeros(batch.S + 1, dtype=np.int64)
+            np.cumsum(counts, out=first[1:])
+            row0 = (np.arange(int(first[-1]), dtype=np.int64) - first[:-1][entry]) * size
+            batch.add_array("latent_tile_entry_%d" % self.heads, entry)
+            batch.add_array("latent_tile_row0_%d" % self.heads, row0)
+            batch.shared[note] = int(first[-1])
+        keys = batch.max_kv_len if self.window is None else min(batch.max_kv_len, self.window + batch.max_q_len - 1)
+        parts = ops.latent_key_parts(batch.shared[note], keys)
+        batch.shared[("latent_parts", self.heads, self.window)] = parts
+        batch.add_graph_key("latent_parts_%d_%s" % (self.heads, self.window), parts)
+
+    def plan_arrays(self, entries):
+        n = entries * -(-self.heads // ops.LATENT_TILE_ROWS)
+        return {"latent_tile_entry_%d" % self.heads: n, "latent_tile_row0_%d" % self.heads: n}
+
     def _frequencies(self):
         if self.position is None:
             return None, 1.0, 0
@@ -107,7 +134,11 @@ class LatentAttention(Mixer):
         else:
             qa[:, :, :r].zero_()
         meta = attention_meta(batch, cache.group, nh)
-        lat = ops.latent_attention(qa, cache.rows, cache.page_size, meta, self.sink, r, self.scale, self.window, x.dtype)
+        tiles, parts = None, 1
+        if ("latent_tiles", nh) in batch.shared:
+            tiles = (batch.array("latent_tile_entry_%d" % nh), batch.array("latent_tile_row0_%d" % nh), batch.shared[("latent_tiles", nh)])
+            parts = batch.shared[("latent_parts", nh, self.window)]
+        lat = ops.latent_attention(qa, cache.rows, cache.page_size, meta, self.sink, r, self.scale, self.window, x.dtype, tiles, parts)
         # the summed latents through the values' expansion: v[t, h, e] = sum_j lat[t, h, j] Wuv[h dv + e, j]
         v = torch.empty((T, nh * dv), dtype=x.dtype, device=x.device)
         ops.gemm_strided(lat, (r, nh * r, 1), self.w_uv, (dv * r, r, 1), v, (dv, nh * dv, 1), nh, T, dv, r)

@@ -33,6 +33,8 @@ def emu_ops(monkeypatch):
     monkeypatch.setattr(ops, "linear_swiglu", lambda x, w, tiled=None: emu.swiglu(emu.linear(x, w)))
     monkeypatch.setattr(ops, "paged_attention", lambda q, k_cache, v_cache, page_size, meta, n_q, n_kv, d, scale, window, raw=None,
                         for_product=False: emu.paged_attention(q, k_cache, v_cache, page_size, meta, n_q, n_kv, d, scale, window))
+    monkeypatch.setattr(ops, "latent_attention", lambda qa, cache, page_size, meta, sink, R, scale, window, out_dtype, tiles=None,
+                        key_parts=1: emu.latent_attention(qa, cache, page_size, meta, sink, R, scale, window, out_dtype))
     monkeypatch.setattr(ops, "tile_weight", lambda w: None)
     monkeypatch.setattr(ops, "fused_decode_ok", lambda *a, **k: False)
     monkeypatch.setattr(ops, "fused_attention_ok", lambda *a, **k: False)

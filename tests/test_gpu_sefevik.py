@@ -125,6 +125,45 @@ def test_mingru_scan_in_pieces_carries_the_state(dtype):
         close(state[slots[e]], s, torch.float32, what="mingru state %d" % e)
 
 
+@pytest.mark.parametrize("case", [dict(H=16, R=512, DR=64, P=16, window=300, entries=[(700, 1), (40, 1), (299, 1), (1500, 1)], parts=6),
+                                  dict(H=16, R=512, DR=64, P=16, window=300, entries=[(0, 350), (811, 5), (64, 1)], parts=1),
+                                  dict(H=5, R=96, DR=32, P=8, window=None, entries=[(0, 70), (130, 3), (257, 1)], parts=3),
+                                  dict(H=72, R=40, DR=8, P=32, window=33, entries=[(100, 1), (0, 45)], parts=2)])
+def test_latent_attention_on_mfma_equals_the_plain_kernel(case):
+    """Rows of real sizes, a sink, a window that begins and ends inside pages and chunks, entries that are single tokens
+    far into a request or portions from its start, keys in parts: against the float32 kernel on the same cache."""
+    import numpy as np
+    from spyinfer_amd.kernels import ops
+    dev = require_gpu()
+    g = torch.Generator().manual_seed(5)
+    H, R, DR, P, window = case["H"], case["R"], case["DR"], case["P"], case["window"]
+    D = R + DR
+    S = len(case["entries"])
+    lens = [n for _, n in case["entries"]]
+    kv = [p0 + n for p0, n in case["entries"]]
+    T = sum(lens)
+    width = max(-(-k // P) for k in kv)
+    pages = sum(-(-k // P) for k in kv) + 3
+    perm = torch.randperm(pages, generator=g).tolist()
+    table = np.full((S, width), -1, dtype=np.int32)
+    for s, k in enumerate(kv):
+        for b in range(-(-k // P)):
+            table[s, b] = perm.pop()
+    cache = torch.randn((pages, P, D), generator=g).to(torch.bfloat16).to(dev)
+    qa = (3.0 * torch.randn((T, H, D), generator=g) / D ** 0.5).to(dev)
+    sink = torch.randn((H,), generator=g).to(torch.bfloat16).to(dev)
+    cu = np.concatenate([[0], np.cumsum(lens)]).astype(np.int32)
+    ent = np.repeat(np.arange(S, dtype=np.int32), lens)
+    pos = np.concatenate([np.arange(p0, p0 + n) for p0, n in case["entries"]]).astype(np.int32)
+    meta = ops.AttentionMeta(i32(cu, dev), i32([p0 for p0, _ in case["entries"]], dev), i32(kv, dev), torch.tensor(table, device=dev),
+                             i32(ent, dev), i32(pos, dev), S, T, width, max(kv), max(lens))
+    counts = [-(-n * H // ops.LATENT_TILE_ROWS) for n in lens]
+    tiles = (i32(np.repeat(np.arange(S), counts), dev), i32(np.concatenate([np.arange(c) * ops.LATENT_TILE_ROWS for c in counts]), dev), sum(counts))
+    ref = ops.latent_attention(qa, cache, P, meta, sink, R, 0.7, window, torch.float32)
+    got = ops.latent_attention(qa, cache, P, meta, sink, R, 0.7, window, torch.bfloat16, tiles, case["parts"])
+    close(got, ref, torch.bfloat16, what="latent attention on MFMA")
+
+
 # ---- whole models under every schedule ------------------------------------------------------------
 MODELS = {"a": (sc.SEF_A, 3, None), "b": (sc.SEF_B, 4, None), "c": (sc.SEF_C, 6, None), "a_sharp": (sc.SEF_A, 5, sc.sharpen()),
           "far_sharp": (sc.SEF_FAR, 8, sc.sharpen(8.0))}
