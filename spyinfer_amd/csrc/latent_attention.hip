@@ -14,8 +14,8 @@
 // ---------------------------------------------------------------------------------------------
 // Rotation: pair (i, i + dims/2), i < dims/2, of the rotated part; angle = position * freq[i] in float32, cos and sin
 // times `mag`.  Values beyond `dims` pass unchanged.
-template <typename TA, typename TW>
-__global__ void latent_prepare_kernel(float* __restrict__ qa, const TA* __restrict__ q, int ldq, const TA* __restrict__ dkv, int ldd,
+template <typename TA, typename TW, typename TQ>
+__global__ void latent_prepare_kernel(TQ* __restrict__ qa, const TA* __restrict__ q, int ldq, const TA* __restrict__ dkv, int ldd,
                                       TA* __restrict__ cache, const int* __restrict__ slot_mapping, long long cache_rows,
                                       const TW* __restrict__ w_norm, float eps, const float* __restrict__ freq, float mag,
                                       int dims, const int* __restrict__ positions, int H, int DN, int DR, int R) {
@@ -35,7 +35,7 @@ __global__ void latent_prepare_kernel(float* __restrict__ qa, const TA* __restri
             const float a = to_f32<TA>(src[j]), b = to_f32<TA>(src[j + half]);
             v = i < half ? a * c - b * s : b * c + a * s;
         }
-        qa[((size_t)t * H + h) * (R + DR) + R + i] = v;
+        qa[((size_t)t * H + h) * (R + DR) + R + i] = from_f32<TQ>(v);
     }
     if (!dkv) return;
     const long long slot = slot_mapping[t];
@@ -60,16 +60,16 @@ __global__ void latent_prepare_kernel(float* __restrict__ qa, const TA* __restri
     }
 }
 
-extern "C" int spy_latent_prepare(float* qa, const void* q, int ldq, const void* dkv, int ldd, int dtype, void* cache,
+extern "C" int spy_latent_prepare(void* qa, int qa_dtype, const void* q, int ldq, const void* dkv, int ldd, int dtype, void* cache,
                                   const int* slot_mapping, long long cache_rows, const void* w_norm, int w_dtype, float eps,
                                   const float* freq, float mag, int dims, const int* positions, int T, int H, int DN, int DR, int R,
                                   hipStream_t st) {
     SPY_REQUIRE(T > 0 && H > 0 && DN >= 0 && DR >= 0 && R > 0, "spy_latent_prepare: empty operand");
     SPY_REQUIRE(dims >= 0 && dims <= DR && dims % 2 == 0 && (dims == 0 || freq), "spy_latent_prepare: %d rotated dims of %d", dims, DR);
     SPY_REQUIRE(!dkv || (cache && slot_mapping && w_norm), "spy_latent_prepare: storing needs the cache, the tokens' slots and the norm weight");
-    SPY_DISPATCH(dtype, TA, SPY_DISPATCH(w_dtype, TW, (latent_prepare_kernel<TA, TW><<<T, 256, 0, st>>>(
-        qa, (const TA*)q, ldq, (const TA*)dkv, ldd, (TA*)cache, slot_mapping, cache_rows, (const TW*)w_norm, eps, freq, mag, dims,
-        positions, H, DN, DR, R))));
+    SPY_DISPATCH(dtype, TA, SPY_DISPATCH(w_dtype, TW, SPY_DISPATCH(qa_dtype, TQ, (latent_prepare_kernel<TA, TW, TQ><<<T, 256, 0, st>>>(
+        (TQ*)qa, (const TA*)q, ldq, (const TA*)dkv, ldd, (TA*)cache, slot_mapping, cache_rows, (const TW*)w_norm, eps, freq, mag, dims,
+        positions, H, DN, DR, R)))));
     SPY_CHECK_LAUNCH("spy_latent_prepare");
     return 0;
 }
@@ -228,7 +228,7 @@ extern "C" int spy_latent_attention(void* out, int out_dtype, const float* qa, c
 // ---------------------------------------------------------------------------------------------
 // The same attention on MFMA for bfloat16 caches.  All heads of a token read the same latent rows, so the query rows of
 // an entry, (token, head) pairs, token major, are one long list against one "kv head": a block of LW waves takes
-// 16 LW consecutive rows (a row tile per wave), walks the keys that its rows' tokens see in chunks of 32, and stages every
+// 16 LW consecutive rows of bfloat16 queries (a row tile per wave), walks the keys that its rows' tokens see in chunks of 32, and stages every
 // chunk in LDS ONCE for all its waves, in two forms: rows [key][D] for S^T = K . Q^T and, for the first R values, the
 // transpose [d][key] for O^T += V^T . P^T (the values are the keys' first part: no second read of memory).  With
 // v_mfma_f32_16x16x32_bf16 tile a of S^T takes keys 8 (r / 4) + r % 4 and tile b those + 4, so that lane (q row, g) holds
@@ -246,7 +246,7 @@ typedef __attribute__((__vector_size__(4 * sizeof(uint32_t)))) uint32_t lu32x4_t
 // QS: most 32-wide steps of D; RT: most 16-wide tiles of R (both bound the registers)
 template <int QS, int RT, typename TW>
 __global__ __launch_bounds__(LW * 64) void latent_attention_mfma_kernel(
-    bf16_t* __restrict__ out, float* __restrict__ ws, const float* __restrict__ qa, const bf16_t* __restrict__ cache, int P,
+    bf16_t* __restrict__ out, float* __restrict__ ws, const bf16_t* __restrict__ qa, const bf16_t* __restrict__ cache, int P,
     int num_pages, const int* __restrict__ cu_q, const int* __restrict__ pos0, const int* __restrict__ kv_len,
     const int* __restrict__ block_table, int max_blocks, const int* __restrict__ tile_entry, const int* __restrict__ tile_row0,
     const TW* __restrict__ sink, int H, int R, int D, float scale, int window) {
@@ -277,15 +277,12 @@ __global__ __launch_bounds__(LW * 64) void latent_attention_mfma_kernel(
     const int lo_row = window > 0 ? prow - window + 1 : 0;
     lbf16x8_t bq[QS];
     {
-        const float* qv = qa + ((size_t)q0 * H + row) * D;
+        const bf16_t* qv = qa + ((size_t)q0 * H + row) * D;
 #pragma unroll
         for (int s = 0; s < QS; ++s) {
             const int d0 = 32 * s + 8 * g;
             lu32x4_t packed = {0u, 0u, 0u, 0u};
-            if (s < q_steps && row_ok && d0 < D) {
-                const float4 x = *reinterpret_cast<const float4*>(qv + d0), y = *reinterpret_cast<const float4*>(qv + d0 + 4);
-                packed = lu32x4_t{pack_bf16x2(x.x, x.y), pack_bf16x2(x.z, x.w), pack_bf16x2(y.x, y.y), pack_bf16x2(y.z, y.w)};
-            }
+            if (s < q_steps && row_ok && d0 < D) packed = *reinterpret_cast<const lu32x4_t*>(qv + d0);
             bq[s] = __builtin_bit_cast(lbf16x8_t, packed);
         }
     }
@@ -301,8 +298,10 @@ __global__ __launch_bounds__(LW * 64) void latent_attention_mfma_kernel(
     for (int c = c_begin; c < c_end; ++c) {
         const int key0 = c_start + 32 * c;
         __syncthreads();                                             // the chunk before is read
+        // a wave's lanes take the 32 keys of two neighbouring 16-byte pieces: the transposed 2-byte stores of a wave then
+        // fall into 16 neighbouring LDS words (lanes along d would all hit one bank)
         for (int i = tid; i < pieces; i += LW * 64) {
-            const int k = i / pieces_per_key, d8 = (i - k * pieces_per_key) * 8;
+            const int k = i & 31, d8 = (i >> 5) * 8;
             const int key = key0 + k;
             lu32x4_t v = {0u, 0u, 0u, 0u};
             if (key >= lo && key <= p_hi && d8 < D) {
@@ -407,17 +406,15 @@ __global__ __launch_bounds__(256) void latent_attention_merge_kernel(bf16_t* __r
     __shared__ float inv_l;
     const size_t row = blockIdx.x;
     const float* base = ws + row * splits * (R + 2);
-    if (threadIdx.x == 0) {
-        float M = -INFINITY;
-        for (int i = 0; i < splits; ++i) M = fmaxf(M, base[(size_t)i * (R + 2) + R]);
-        float L = 0.f;
-        for (int i = 0; i < splits; ++i) {
-            const float mi = base[(size_t)i * (R + 2) + R];
-            const float e = (mi == -INFINITY) ? 0.f : expf(mi - M);
-            wgt[i] = e;
-            L += base[(size_t)i * (R + 2) + R + 1] * e;
-        }
-        inv_l = L > 0.f ? 1.0f / L : 0.f;
+    if (threadIdx.x < 64) {                        // the parts' maxima and sums, one lane each (at most 64 parts)
+        const int i = threadIdx.x;
+        const float mi = i < splits ? base[(size_t)i * (R + 2) + R] : -INFINITY;
+        const float li = i < splits ? base[(size_t)i * (R + 2) + R + 1] : 0.f;
+        const float M = wave_max(mi);
+        const float e = (mi == -INFINITY) ? 0.f : __expf(mi - M);
+        wgt[i] = e;
+        const float L = wave_sum(li * e);
+        if (i == 0) inv_l = L > 0.f ? 1.0f / L : 0.f;
     }
     __syncthreads();
     for (int j = threadIdx.x; j < R; j += blockDim.x) {
@@ -432,7 +429,7 @@ extern "C" long long spy_latent_attention_mfma_workspace(int T, int H, int R, in
 }
 
 // tiles: num_tiles records (entry, first row) of 64 rows each.  ws: float32, spy_latent_attention_mfma_workspace values.
-extern "C" int spy_latent_attention_mfma(void* out, float* ws, const float* qa, const void* cache, int P, int num_pages,
+extern "C" int spy_latent_attention_mfma(void* out, float* ws, const void* qa, const void* cache, int P, int num_pages,
                                          const int* cu_q, const int* pos0, const int* kv_len, const int* block_table,
                                          int max_blocks, const int* tile_entry, const int* tile_row0, int num_tiles,
                                          const void* sink, int sink_dtype, int T, int H, int R, int DR, float scale, int window,
@@ -453,7 +450,7 @@ extern "C" int spy_latent_attention_mfma(void* out, float* ws, const float* qa, 
             hipError_t e_ = hipFuncSetAttribute((const void*)kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);      \
             if (e_ != hipSuccess) return spy_fail("spy_latent_attention_mfma: %zu bytes of LDS refused: %s", lds, hipGetErrorString(e_)); \
         }                                                                                                                       \
-        kernel<<<grid, LW * 64, lds, st>>>((bf16_t*)out, ws, qa, (const bf16_t*)cache, P, num_pages, cu_q, pos0, kv_len,        \
+        kernel<<<grid, LW * 64, lds, st>>>((bf16_t*)out, ws, (const bf16_t*)qa, (const bf16_t*)cache, P, num_pages, cu_q, pos0, kv_len,        \
                                            block_table, max_blocks, tile_entry, tile_row0, (const TW*)sink, H, R, D, scale, window); \
     })
     if (q_steps <= 8 && r_tiles <= 8) { SPY_LA_LAUNCH(8, 8); }
@@ -462,8 +459,64 @@ extern "C" int spy_latent_attention_mfma(void* out, float* ws, const float* qa, 
 #undef SPY_LA_LAUNCH
     SPY_CHECK_LAUNCH("spy_latent_attention_mfma");
     if (splits > 1) {
-        latent_attention_merge_kernel<<<(unsigned)((size_t)T * H), R >= 256 ? 256 : 64, 0, st>>>((bf16_t*)out, ws, R, splits);
+        latent_attention_merge_kernel<<<(unsigned)((size_t)T * H), R > 128 ? 256 : 64, 0, st>>>((bf16_t*)out, ws, R, splits);
         SPY_CHECK_LAUNCH("spy_latent_attention_mfma (merge)");
     }
+    return 0;
+}
+
+// ---------------------------------------------------------------------------------------------
+// Per-head products of few rows on MFMA: C[t, h, n] = sum_k X[t, h, k] W[h, n, k], bfloat16 operands with k innermost
+// (X with element strides between tokens and heads, W [H][N][K] in one piece), float32 sums.  A wave owns 16 columns n
+// of one head, holds their part of W in registers (KS steps of 32 k values) and walks the tokens in tiles of 16: W is
+// read once.  This is the step of single tokens' form of the products with the keys' and the values' expansion matrices;
+// many rows take the library's batched product.
+template <int KS, typename TC>
+__global__ __launch_bounds__(256) void head_products_kernel(TC* __restrict__ C, long long ct, long long ch, const bf16_t* __restrict__ X,
+                                                            long long xt, long long xh, const bf16_t* __restrict__ W, int T, int N, int K) {
+    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63, r16 = lane & 15, g = lane >> 4;
+    const int n0 = (blockIdx.x * 4 + wave) * 16, h = blockIdx.y;
+    if (n0 >= N) return;
+    lbf16x8_t wr[KS];
+    const int n = n0 + r16;
+#pragma unroll
+    for (int s = 0; s < KS; ++s) {
+        const int k0 = 32 * s + 8 * g;
+        lu32x4_t v = {0u, 0u, 0u, 0u};
+        if (n < N && k0 < K) v = *reinterpret_cast<const lu32x4_t*>(W + ((size_t)h * N + n) * K + k0);
+        wr[s] = __builtin_bit_cast(lbf16x8_t, v);
+    }
+    for (int t0 = blockIdx.z * 16; t0 < T; t0 += gridDim.z * 16) {
+        const int t = t0 + r16;
+        lf32x4_t acc = {0.f, 0.f, 0.f, 0.f};
+        const bf16_t* x = X + (size_t)t * xt + (size_t)h * xh;
+#pragma unroll
+        for (int s = 0; s < KS; ++s) {
+            const int k0 = 32 * s + 8 * g;
+            lu32x4_t v = {0u, 0u, 0u, 0u};
+            if (t < T && k0 < K) v = *reinterpret_cast<const lu32x4_t*>(x + k0);
+            acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wr[s], __builtin_bit_cast(lbf16x8_t, v), acc, 0, 0, 0);
+        }
+        // lane (t = r16, g) holds C[t][h][n0 + 4 g + j], j < 4
+        if (t < T) {
+            TC* c = C + (size_t)t * ct + (size_t)h * ch + n0 + 4 * g;
+#pragma unroll
+            for (int j = 0; j < 4; ++j)
+                if (n0 + 4 * g + j < N) c[j] = from_f32<TC>(acc[j]);
+        }
+    }
+}
+
+extern "C" int spy_head_products(void* C, int c_dtype, long long ct, long long ch, const void* X, long long xt, long long xh,
+                                 const void* W, int T, int H, int N, int K, hipStream_t st) {
+    SPY_REQUIRE(T > 0 && H > 0 && N > 0 && K > 0 && H <= 65535, "spy_head_products: empty operand");
+    SPY_REQUIRE(K % 8 == 0 && K <= 512 && xt % 8 == 0 && xh % 8 == 0 && ((uintptr_t)X % 16) == 0 && ((uintptr_t)W % 16) == 0,
+                "spy_head_products: K = %d (a multiple of 8 up to 512) and 16-byte pieces of the operands expected", K);
+    const int t_tiles = (T + 15) / 16;
+    const dim3 grid((N + 63) / 64, H, t_tiles < 8 ? t_tiles : 8);
+#define SPY_HP_LAUNCH(KS) SPY_DISPATCH(c_dtype, TC, (head_products_kernel<KS, TC><<<grid, 256, 0, st>>>((TC*)C, ct, ch, (const bf16_t*)X, xt, xh, (const bf16_t*)W, T, N, K)))
+    if (K <= 128) { SPY_HP_LAUNCH(4); } else if (K <= 256) { SPY_HP_LAUNCH(8); } else { SPY_HP_LAUNCH(16); }
+#undef SPY_HP_LAUNCH
+    SPY_CHECK_LAUNCH("spy_head_products");
     return 0;
 }

@@ -76,7 +76,7 @@ class _Hip:
                      "spy_sample", "spy_sample_workspace", "spy_gemm_skinny", "spy_gemm_skinny_swiglu",
                      "spy_gemm_decode", "spy_gemm_decode_workspace", "spy_embedding_sumsq", "spy_sample_static", "spy_measure_read",
                      "spy_pair_embedding", "spy_norm_residual", "spy_depth_mix", "spy_xielu", "spy_mingru", "spy_latent_prepare",
-                     "spy_gemm_strided", "spy_latent_attention", "spy_latent_attention_mfma", "spy_latent_attention_mfma_workspace"):
+                     "spy_gemm_strided", "spy_latent_attention", "spy_latent_attention_mfma", "spy_latent_attention_mfma_workspace", "spy_head_products"):
             if not hasattr(self.lib, name):
                 raise KernelError("the kernel library %s lacks %s: it is older than its sources; build it again "
                                   "(spyinfer_amd.kernels.build.build())" % (self.lib._name, name))
@@ -977,11 +977,11 @@ def gemm_strided(a: torch.Tensor, a_strides, b: torch.Tensor, b_strides, c: torc
 
 def latent_prepare(q: torch.Tensor, dkv: Optional[torch.Tensor], cache: Optional[torch.Tensor], slot_mapping: Optional[torch.Tensor],
                    w_norm: Optional[torch.Tensor], eps: float, freq: Optional[torch.Tensor], mag: float, dims: int,
-                   positions: torch.Tensor, H: int, DN: int, DR: int, R: int) -> torch.Tensor:
+                   positions: torch.Tensor, H: int, DN: int, DR: int, R: int, qa_dtype: torch.dtype = torch.float32) -> torch.Tensor:
     """Queries ``q [T, >= H (DN + DR)]`` (a row may be a view into a wider product: its stride is taken) and, if given,
     ``dkv [T, >= R + DR]``: the latent rmsnorm(dkv[:R]) * w_norm and the rotated dkv[R:] go to ``cache [pages, P, R + DR]``
-    at the tokens' slots; returns the absorbed query rows float32 [T, H, R + DR] with the rotated part filled in (the
-    first R values of a row are for the caller's product with the keys' expansion matrix)."""
+    at the tokens' slots; returns the absorbed query rows [T, H, R + DR] in ``qa_dtype`` with the rotated part filled in
+    (the first R values of a row are for the caller's product with the keys' expansion matrix)."""
     _check(q.dim() == 2 and q.stride(1) == 1 and q.is_cuda, "latent_prepare: q must be rows on the GPU")
     T = q.shape[0]
     _check(q.shape[1] >= H * (DN + DR), "latent_prepare: q rows hold %d values, %d heads of %d needed", q.shape[1], H, DN + DR)
@@ -998,9 +998,9 @@ def latent_prepare(q: torch.Tensor, dkv: Optional[torch.Tensor], cache: Optional
         _check(slot_mapping is not None and slot_mapping.dtype == torch.int32 and slot_mapping.shape == (T,) and w_norm is not None
                and w_norm.shape == (R,), "latent_prepare: slot_mapping int32 [T] and a norm weight [R] expected")
         rows = cache.shape[0] * cache.shape[1]
-    qa = torch.empty((T, H, R + DR), dtype=torch.float32, device=q.device)
+    qa = torch.empty((T, H, R + DR), dtype=qa_dtype, device=q.device)
     if T:
-        hip().call("spy_latent_prepare", _ptr(qa), ctypes.c_void_p(q.data_ptr()), ctypes.c_int(q.stride(0)),
+        hip().call("spy_latent_prepare", _ptr(qa), _code(qa, "qa"), ctypes.c_void_p(q.data_ptr()), ctypes.c_int(q.stride(0)),
                    ctypes.c_void_p(0 if dkv is None else dkv.data_ptr()), ctypes.c_int(0 if dkv is None else dkv.stride(0)),
                    _code(q, "q"), _ptr(cache if dkv is not None else None), _ptr(slot_mapping if dkv is not None else None),
                    ctypes.c_longlong(rows), _ptr(w_norm if dkv is not None else None),
@@ -1010,6 +1010,33 @@ def latent_prepare(q: torch.Tensor, dkv: Optional[torch.Tensor], cache: Optional
     return qa
 
 
+def head_products_ok(x: torch.Tensor, xt: int, xh: int, K: int) -> bool:
+    """Whether ``head_products`` takes these operands."""
+    return x.dtype == torch.bfloat16 and K % 8 == 0 and 0 < K <= 512 and xt % 8 == 0 and xh % 8 == 0 and x.data_ptr() % 16 == 0
+
+
+def head_products(x: torch.Tensor, xt: int, xh: int, w: torch.Tensor, out: torch.Tensor, ct: int, ch: int, T: int) -> torch.Tensor:
+    """out[t, h, n] = sum_k x[t, h, k] * w[h, n, k] on MFMA: ``w [H, N, K]`` bfloat16 in one piece, ``x`` bfloat16 with
+    element strides (xt between tokens, xh between heads, k innermost), ``out`` float32 or bfloat16 with strides (ct, ch).
+    Built for few rows (a wave keeps its part of ``w`` in registers and walks the tokens)."""
+    _check(x.is_cuda and out.is_cuda and x.device == out.device, "head_products: operands on one GPU expected")
+    _dev(w)
+    _check(w.dim() == 3 and w.dtype == torch.bfloat16, "head_products: w must be bfloat16 [H, N, K]")
+    H, N, K = w.shape
+    _check(head_products_ok(x, xt, xh, K), "head_products: x must be bfloat16 in 16-byte pieces, K a multiple of 8 up to 512")
+    _check((T - 1) * xt + (H - 1) * xh + K <= x.untyped_storage().nbytes() // 2 - x.storage_offset(), "head_products: x's strides reach beyond it")
+    _check((T - 1) * ct + (H - 1) * ch + N <= out.untyped_storage().nbytes() // out.element_size() - out.storage_offset(),
+           "head_products: out's strides reach beyond it")
+    if T:
+        hip().call("spy_head_products", ctypes.c_void_p(out.data_ptr()), _code(out, "out"), ctypes.c_longlong(ct), ctypes.c_longlong(ch),
+                   ctypes.c_void_p(x.data_ptr()), ctypes.c_longlong(xt), ctypes.c_longlong(xh), _ptr(w), ctypes.c_int(T), ctypes.c_int(H),
+                   ctypes.c_int(N), ctypes.c_int(K), _Hip.stream())
+    return out
+
+
+#: most rows of a step for which the per-head products of the latent attention run on ``head_products``; more rows take
+#: the library's batched product
+HEAD_PRODUCTS_MAX_ROWS = 128
 LATENT_TILE_ROWS = 64       # query rows, (token, head) pairs, of one block of the MFMA latent attention
 LATENT_MFMA = True          # False forces the plain kernel for bfloat16 too (tests flip it; nothing else does)
 
@@ -1028,18 +1055,21 @@ def latent_key_parts(num_tiles: int, max_keys: int) -> int:
 
 def latent_attention(qa: torch.Tensor, cache: torch.Tensor, page_size: int, meta: "AttentionMeta", sink: Optional[torch.Tensor],
                      R: int, scale: float, window: Optional[int], out_dtype: torch.dtype, tiles=None, key_parts: int = 1) -> torch.Tensor:
-    """Attention of ``qa [T, H, R + DR]`` (float32, absorbed queries) over the latent rows ``cache [pages, P, R + DR]``:
+    """Attention of ``qa [T, H, R + DR]`` (absorbed queries: float32 for the plain kernel, bfloat16 with ``tiles`` for the
+    MFMA kernel) over the latent rows ``cache [pages, P, R + DR]``:
     score = qa . row * scale, softmax with exp(sink[h]) added to the denominator, causal with ``window``; the result is
     sum_j p_j row_j[:R], [T, H, R] in ``out_dtype``."""
     _dev(qa, cache, sink, meta.kv_len, meta.block_table, meta.token_entry, meta.positions)
-    _check(qa.dtype == torch.float32 and qa.dim() == 3, "latent_attention: qa must be float32 [T, H, D]")
+    _check(qa.dim() == 3, "latent_attention: qa must be [T, H, D]")
     T, H, D = qa.shape
+    mfma = tiles is not None and out_dtype == torch.bfloat16 and latent_attention_mfma_ok(cache.dtype, R, D)
+    _check(qa.dtype == (torch.bfloat16 if mfma else torch.float32), "latent_attention: query rows are bfloat16 for the MFMA kernel, float32 for the plain one")
     _check(T == meta.T and cache.dim() == 3 and cache.shape[1] == page_size and cache.shape[2] == D and 0 < R <= D,
            "latent_attention: cache [pages, P, %d] expected for %d tokens", D, meta.T)
     _check(sink is None or sink.shape == (H,), "latent_attention: one sink per head expected")
     _check(meta.block_table.shape == (meta.S, meta.max_blocks), "latent_attention: block table must be [S, max_blocks]")
     out = torch.empty((T, H, R), dtype=out_dtype, device=qa.device)
-    if T and tiles is not None and out_dtype == torch.bfloat16 and latent_attention_mfma_ok(cache.dtype, R, D):
+    if T and mfma:
         # tiles: (entry [n], first row [n], n) of LATENT_TILE_ROWS rows each, planned on the host
         tile_entry, tile_row0, n = tiles
         _dev(tile_entry, tile_row0, meta.cu_q, meta.pos0)

@@ -70,7 +70,11 @@ class LatentAttention(Mixer):
             w_in = torch.cat([w_q, w_d], dim=0).contiguous()          # one product: rows [q of all heads | dkv]
             self.c_norm = weights[dkv_norm]
         self.w_in, self.w_in_tiled = ops.weight_forms(w_in)
-        self.w_uk, self.w_uv = weights.pop(uk), weights.pop(uv)
+        nh, dn, dv, r = self.heads, self.dim, self.vdim, self.kv_rank
+        # both expansion matrices per head with the summed index innermost: [H, kv_rank, dim] (transposed once, here) for
+        # the queries' way through the keys' expansion, [H, vdim, kv_rank] (as stored) for the summed latents' way out
+        self.w_uk = weights.pop(uk).view(nh, dn, r).transpose(1, 2).contiguous()
+        self.w_uv = weights.pop(uv).view(nh, dv, r).contiguous()
         self.w_o, self.w_o_tiled = ops.weight_forms(weights.pop(o))
         if self.has_sink:
             self.sink = weights[sink]
@@ -125,21 +129,34 @@ class LatentAttention(Mixer):
         qd = ops.linear(x, self.w_in, tiled=self.w_in_tiled)
         nq = nh * (dn + dr)
         freq, mag, dims = self._frequencies()
+        mfma = ("latent_tiles", nh) in batch.shared            # planned: the MFMA kernel takes these rows (bfloat16 queries)
         qa = ops.latent_prepare(qd, qd[:, nq:] if store else None, cache.rows if store else None,
                                 batch.slot_mapping(cache.group) if store else None, self.c_norm, self.norm_eps, freq, mag, dims,
-                                batch.positions, nh, dn, dr, r)
+                                batch.positions, nh, dn, dr, r, torch.bfloat16 if mfma else torch.float32)
+        D, ld = r + dr, qd.stride(0)
+        library = mfma and T > ops.HEAD_PRODUCTS_MAX_ROWS and self.w_uk.dtype == torch.bfloat16
         # the unrotated query parts through the keys' expansion: qa[t, h, :r] = sum_d q[t, h, d] Wuk[h dn + d, :]
-        if dn:
-            ops.gemm_strided(qd, (dn + dr, qd.stride(0), 1), self.w_uk, (dn * r, 1, r), qa, (r + dr, nh * (r + dr), 1), nh, T, r, dn)
-        else:
+        if not dn:
             qa[:, :, :r].zero_()
+        elif library:
+            qa[:, :, :r].copy_(torch.bmm(qd[:, :nq].unflatten(1, (nh, dn + dr))[:, :, :dn].transpose(0, 1), self.w_uk.transpose(1, 2)).transpose(0, 1))
+        elif mfma and self.w_uk.dtype == torch.bfloat16 and ops.head_products_ok(qd, ld, dn + dr, dn):
+            ops.head_products(qd, ld, dn + dr, self.w_uk, qa, nh * D, D, T)
+        else:
+            ops.gemm_strided(qd, (dn + dr, ld, 1), self.w_uk, (r * dn, dn, 1), qa, (D, nh * D, 1), nh, T, r, dn)
         meta = attention_meta(batch, cache.group, nh)
         tiles, parts = None, 1
-        if ("latent_tiles", nh) in batch.shared:
+        if mfma:
             tiles = (batch.array("latent_tile_entry_%d" % nh), batch.array("latent_tile_row0_%d" % nh), batch.shared[("latent_tiles", nh)])
             parts = batch.shared[("latent_parts", nh, self.window)]
         lat = ops.latent_attention(qa, cache.rows, cache.page_size, meta, self.sink, r, self.scale, self.window, x.dtype, tiles, parts)
         # the summed latents through the values' expansion: v[t, h, e] = sum_j lat[t, h, j] Wuv[h dv + e, j]
-        v = torch.empty((T, nh * dv), dtype=x.dtype, device=x.device)
-        ops.gemm_strided(lat, (r, nh * r, 1), self.w_uv, (dv * r, r, 1), v, (dv, nh * dv, 1), nh, T, dv, r)
+        if library and self.w_uv.dtype == torch.bfloat16:
+            v = torch.bmm(lat.transpose(0, 1), self.w_uv.transpose(1, 2)).transpose(0, 1).reshape(T, nh * dv)
+        else:
+            v = torch.empty((T, nh * dv), dtype=x.dtype, device=x.device)
+            if self.w_uv.dtype == torch.bfloat16 and ops.head_products_ok(lat, nh * r, r, r):
+                ops.head_products(lat, nh * r, r, self.w_uv, v, nh * dv, dv, T)
+            else:
+                ops.gemm_strided(lat, (r, nh * r, 1), self.w_uv, (dv * r, r, 1), v, (dv, nh * dv, 1), nh, T, dv, r)
         return ops.linear(v, self.w_o, tiled=self.w_o_tiled)

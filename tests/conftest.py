@@ -35,6 +35,7 @@ def emu_ops(monkeypatch):
                         for_product=False: emu.paged_attention(q, k_cache, v_cache, page_size, meta, n_q, n_kv, d, scale, window))
     monkeypatch.setattr(ops, "latent_attention", lambda qa, cache, page_size, meta, sink, R, scale, window, out_dtype, tiles=None,
                         key_parts=1: emu.latent_attention(qa, cache, page_size, meta, sink, R, scale, window, out_dtype))
+    monkeypatch.setattr(ops, "latent_attention_mfma_ok", lambda dtype, R, D: False)
     monkeypatch.setattr(ops, "tile_weight", lambda w: None)
     monkeypatch.setattr(ops, "fused_decode_ok", lambda *a, **k: False)
     monkeypatch.setattr(ops, "fused_attention_ok", lambda *a, **k: False)

@@ -180,7 +180,7 @@ class EmuOps:
         a, b = v[..., :half], v[..., half:dims]
         return torch.cat([a * c - b * s, b * c + a * s, v[..., dims:]], dim=-1)
 
-    def latent_prepare(self, q, dkv, cache, slot_mapping, w_norm, eps, freq, mag, dims, positions, H, DN, DR, R):
+    def latent_prepare(self, q, dkv, cache, slot_mapping, w_norm, eps, freq, mag, dims, positions, H, DN, DR, R, qa_dtype=torch.float32):
         T = q.shape[0]
         qa = torch.zeros((T, H, R + DR), dtype=torch.float32)
         qh = q[:, :H * (DN + DR)].float().reshape(T, H, DN + DR)

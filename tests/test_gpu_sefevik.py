@@ -160,8 +160,23 @@ def test_latent_attention_on_mfma_equals_the_plain_kernel(case):
     counts = [-(-n * H // ops.LATENT_TILE_ROWS) for n in lens]
     tiles = (i32(np.repeat(np.arange(S), counts), dev), i32(np.concatenate([np.arange(c) * ops.LATENT_TILE_ROWS for c in counts]), dev), sum(counts))
     ref = ops.latent_attention(qa, cache, P, meta, sink, R, 0.7, window, torch.float32)
-    got = ops.latent_attention(qa, cache, P, meta, sink, R, 0.7, window, torch.bfloat16, tiles, case["parts"])
+    got = ops.latent_attention(qa.to(torch.bfloat16), cache, P, meta, sink, R, 0.7, window, torch.bfloat16, tiles, case["parts"])
     close(got, ref, torch.bfloat16, what="latent attention on MFMA")
+
+
+@pytest.mark.parametrize("T,H,N,K,out_dtype", [(1, 16, 512, 128, torch.bfloat16), (37, 3, 40, 72, torch.float32), (128, 8, 128, 512, torch.bfloat16)])
+def test_head_products(T, H, N, K, out_dtype):
+    from spyinfer_amd.kernels import ops
+    dev = require_gpu()
+    g = torch.Generator().manual_seed(6)
+    pad = 24                                              # the rows of x are views into wider rows
+    x = torch.randn((T, H * (K + pad)), generator=g).to(torch.bfloat16).to(dev)
+    w = (torch.randn((H, N, K), generator=g) / K ** 0.5).to(torch.bfloat16).to(dev)
+    out = torch.zeros((T, H, N + 4), dtype=out_dtype, device=dev)
+    ops.head_products(x, H * (K + pad), K + pad, w, out, H * (N + 4), N + 4, T)
+    ref = torch.einsum("thk,hnk->thn", x.view(T, H, K + pad)[:, :, :K].double().cpu(), w.double().cpu())
+    close(out[:, :, :N], ref, out_dtype if out_dtype == torch.bfloat16 else torch.float32, what="head_products")
+    assert float(out[:, :, N:].abs().max()) == 0.0
 
 
 # ---- whole models under every schedule ------------------------------------------------------------
