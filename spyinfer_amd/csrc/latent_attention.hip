@@ -229,7 +229,7 @@ extern "C" int spy_latent_attention(void* out, int out_dtype, const float* qa, c
 // The same attention on MFMA for bfloat16 caches.  All heads of a token read the same latent rows, so the query rows of
 // an entry, (token, head) pairs, token major, are one long list against one "kv head": a block of LW waves takes
 // 16 LW consecutive rows of bfloat16 queries (a row tile per wave), walks the keys that its rows' tokens see in chunks of 32, and stages every
-// chunk in LDS ONCE for all its waves, in two forms: rows [key][D] for S^T = K . Q^T and, for the first R values, the
+// chunk in LDS ONCE for all its waves (two buffers in turn), in two forms: rows [key][D] for S^T = K . Q^T and, for the first R values, the
 // transpose [d][key] for O^T += V^T . P^T (the values are the keys' first part: no second read of memory).  With
 // v_mfma_f32_16x16x32_bf16 tile a of S^T takes keys 8 (r / 4) + r % 4 and tile b those + 4, so that lane (q row, g) holds
 // the scores of keys 8 g .. 8 g + 7, exactly the 8 k values of its P^T operand.  Softmax float32, online, the sink in
@@ -268,8 +268,7 @@ __global__ __launch_bounds__(LW * 64) void latent_attention_mfma_kernel(
     const int c_begin = (int)((long long)n_chunks * sp / splits), c_end = (int)((long long)n_chunks * (sp + 1) / splits);
     const int q_steps = (D + 31) / 32, r_tiles = (R + 15) / 16;
     const int Dp = q_steps * 32, krow = Dp + LKPAD;
-    bf16_t* Ks = reinterpret_cast<bf16_t*>(lds_raw);                  // [32][krow]
-    bf16_t* Vt = Ks + 32 * krow;                                       // [r_tiles * 16][LVROW]
+    bf16_t* Ks = reinterpret_cast<bf16_t*>(lds_raw);                  // two buffers of { keys [32][krow], values [r_tiles * 16][LVROW] }
     // this lane's query row
     const int row = r_lo + 16 * wave + r16;
     const bool row_ok = row <= r_hi;
@@ -293,38 +292,67 @@ __global__ __launch_bounds__(LW * 64) void latent_attention_mfma_kernel(
 #pragma unroll
     for (int i = 0; i < RT; ++i) acc[i] = lf32x4_t{0.f, 0.f, 0.f, 0.f};
     const int* bt = block_table + (size_t)e * max_blocks;
-    const int pieces_per_key = Dp / 8, pieces = 32 * pieces_per_key;
     const int ka_row = 8 * (r16 >> 2) + (r16 & 3);                  // tile a's key of this lane's operand row; tile b: + 4
-    for (int c = c_begin; c < c_end; ++c) {
-        const int key0 = c_start + 32 * c;
-        __syncthreads();                                             // the chunk before is read
-        // a wave's lanes take the 32 keys of two neighbouring 16-byte pieces: the transposed 2-byte stores of a wave then
-        // fall into 16 neighbouring LDS words (lanes along d would all hit one bank)
-        for (int i = tid; i < pieces; i += LW * 64) {
-            const int k = i & 31, d8 = (i >> 5) * 8;
-            const int key = key0 + k;
-            lu32x4_t v = {0u, 0u, 0u, 0u};
-            if (key >= lo && key <= p_hi && d8 < D) {
-                const int page = bt[key / P];
-                if (page >= 0 && page < num_pages) v = *reinterpret_cast<const lu32x4_t*>(cache + ((size_t)page * P + key % P) * D + d8);
-            }
-            *reinterpret_cast<lu32x4_t*>(Ks + k * krow + d8) = v;
-            if (d8 < r_tiles * 16) {
+    // Staging.  A thread takes ONE key of a chunk (tid % 32) and every eighth 16-byte piece of its row: a wave's lanes are
+    // the 32 keys of two neighbouring pieces, so its transposed 2-byte stores fall into 16 neighbouring LDS words (lanes
+    // along d would all hit one bank), and a thread looks up one page per chunk.  The pieces of chunk c + 2 are asked for
+    // (into registers) before chunk c is multiplied, and chunk c + 1 is written to the second LDS buffer before that: one
+    // barrier per chunk, and no wave waits for memory while another has products to do.
+    constexpr int NP = (QS + 1) / 2;
+    const int sk = tid & 31, sd0 = (tid >> 5) * 8;
+    const int buf_elems = 32 * krow + r_tiles * 16 * LVROW;
+    lu32x4_t pf[NP];
+    auto fetch = [&](int c) {
+        const int key = c_start + 32 * c + sk;
+        const bf16_t* src = nullptr;
+        if (c < c_end && key >= lo && key <= p_hi) {
+            const int page = bt[key / P];
+            if (page >= 0 && page < num_pages) src = cache + ((size_t)page * P + key % P) * D;
+        }
 #pragma unroll
-                for (int j = 0; j < 4; ++j) {
-                    Vt[(d8 + 2 * j) * LVROW + k] = (bf16_t)(v[j] & 0xffffu);
-                    Vt[(d8 + 2 * j + 1) * LVROW + k] = (bf16_t)(v[j] >> 16);
+        for (int it = 0; it < NP; ++it) {
+            const int d8 = sd0 + 64 * it;
+            pf[it] = lu32x4_t{0u, 0u, 0u, 0u};
+            if (src && d8 < D) pf[it] = *reinterpret_cast<const lu32x4_t*>(src + d8);
+        }
+    };
+    auto stage = [&](int c) {
+        bf16_t* ks = Ks + (c & 1) * buf_elems;
+        bf16_t* vt = ks + 32 * krow;
+#pragma unroll
+        for (int it = 0; it < NP; ++it) {
+            const int d8 = sd0 + 64 * it;
+            if (d8 < Dp) {
+                *reinterpret_cast<lu32x4_t*>(ks + sk * krow + d8) = pf[it];
+                if (d8 < r_tiles * 16) {
+#pragma unroll
+                    for (int j = 0; j < 4; ++j) {
+                        vt[(d8 + 2 * j) * LVROW + sk] = (bf16_t)(pf[it][j] & 0xffffu);
+                        vt[(d8 + 2 * j + 1) * LVROW + sk] = (bf16_t)(pf[it][j] >> 16);
+                    }
                 }
             }
         }
-        __syncthreads();
+    };
+    if (c_begin < c_end) {
+        fetch(c_begin);
+        stage(c_begin);
+        fetch(c_begin + 1);
+    }
+    __syncthreads();
+    for (int c = c_begin; c < c_end; ++c) {
+        const int key0 = c_start + 32 * c;
+        if (c + 1 < c_end) stage(c + 1);                             // into the buffer that chunk c - 1 was read from, before the barrier below
+        fetch(c + 2);
+        const bf16_t* Kc = Ks + (c & 1) * buf_elems;
+        const bf16_t* Vc = Kc + 32 * krow;
         // ---- S^T = K . Q^T ----
         lf32x4_t sa = {0.f, 0.f, 0.f, 0.f}, sb = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
         for (int s = 0; s < QS; ++s) {
             if (s < q_steps) {
-                const lbf16x8_t ka = *reinterpret_cast<const lbf16x8_t*>(Ks + ka_row * krow + 32 * s + 8 * g);
-                const lbf16x8_t kb = *reinterpret_cast<const lbf16x8_t*>(Ks + (ka_row + 4) * krow + 32 * s + 8 * g);
+                const lbf16x8_t ka = *reinterpret_cast<const lbf16x8_t*>(Kc + ka_row * krow + 32 * s + 8 * g);
+                const lbf16x8_t kb = *reinterpret_cast<const lbf16x8_t*>(Kc + (ka_row + 4) * krow + 32 * s + 8 * g);
                 sa = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ka, bq[s], sa, 0, 0, 0);
                 sb = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kb, bq[s], sb, 0, 0, 0);
             }
@@ -361,11 +389,12 @@ __global__ __launch_bounds__(LW * 64) void latent_attention_mfma_kernel(
 #pragma unroll
         for (int i = 0; i < RT; ++i) {
             if (i < r_tiles) {
-                const lbf16x8_t vt = *reinterpret_cast<const lbf16x8_t*>(Vt + (16 * i + r16) * LVROW + 8 * g);
+                const lbf16x8_t vt = *reinterpret_cast<const lbf16x8_t*>(Vc + (16 * i + r16) * LVROW + 8 * g);
                 acc[i] *= alpha;
                 acc[i] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vt, pb, acc[i], 0, 0, 0);
             }
         }
+        __syncthreads();                                             // chunk c is read by all, chunk c + 1 is written by all
     }
     // the row's sum over its four lanes
     l += __shfl_xor(l, 16, 64);
@@ -437,11 +466,12 @@ extern "C" int spy_latent_attention_mfma(void* out, float* ws, const void* qa, c
     const int D = R + DR;
     SPY_REQUIRE(T > 0 && H > 0 && R > 0 && DR >= 0 && P > 0 && num_pages > 0 && max_blocks > 0 && num_tiles > 0,
                 "spy_latent_attention_mfma: empty operand");
-    SPY_REQUIRE(D % 8 == 0 && R % 8 == 0 && D <= 640 && R <= 512, "spy_latent_attention_mfma: rows of %d + %d values are not taken", R, DR);
+    SPY_REQUIRE(D % 8 == 0 && R % 8 == 0 && D <= 576 && R <= 512, "spy_latent_attention_mfma: rows of %d + %d values are not taken", R, DR);
     SPY_REQUIRE(splits >= 1 && splits <= 64 && (splits == 1 || ws), "spy_latent_attention_mfma: %d parts (1..64, with a workspace)", splits);
     SPY_REQUIRE(((uintptr_t)qa % 16) == 0 && ((uintptr_t)cache % 16) == 0 && ((uintptr_t)out % 8) == 0, "spy_latent_attention_mfma: operands are not aligned");
     const int q_steps = (D + 31) / 32, r_tiles = (R + 15) / 16;
-    const size_t lds = ((size_t)32 * (q_steps * 32 + LKPAD) + (size_t)r_tiles * 16 * LVROW) * sizeof(bf16_t);
+    const size_t lds = 2 * ((size_t)32 * (q_steps * 32 + LKPAD) + (size_t)r_tiles * 16 * LVROW) * sizeof(bf16_t);
+    SPY_REQUIRE(lds <= 160 * 1024, "spy_latent_attention_mfma: two staged chunks of %d + %d values take %zu bytes of LDS", R, DR, lds);
     const dim3 grid(num_tiles, splits);
 #define SPY_LA_LAUNCH(QS, RT)                                                                                                   \
     SPY_DISPATCH(sink_dtype, TW, {                                                                                              \
@@ -455,7 +485,7 @@ extern "C" int spy_latent_attention_mfma(void* out, float* ws, const void* qa, c
     })
     if (q_steps <= 8 && r_tiles <= 8) { SPY_LA_LAUNCH(8, 8); }
     else if (q_steps <= 12 && r_tiles <= 16) { SPY_LA_LAUNCH(12, 16); }
-    else { SPY_LA_LAUNCH(20, 32); }
+    else { SPY_LA_LAUNCH(18, 32); }
 #undef SPY_LA_LAUNCH
     SPY_CHECK_LAUNCH("spy_latent_attention_mfma");
     if (splits > 1) {

@@ -82,9 +82,14 @@ extern "C" int spy_pair_embedding(float* out, void* copy, int copy_dtype, const 
 // ---------------------------------------------------------------------------------------------
 // out[t] = base[t] + y[t] / sqrt(mean(y[t]^2) + eps) * w;  copy[t] (optional) = the same in the activation dtype.
 // out may be base (in place).  One block per row; y is read twice (the second read comes from the cache).
+// With `mix` (n weights): out[t] is one of n kept layer results, kept[n - 1][t], and the kernel also writes
+// mixed[t] = sum over j < n of mix[j] * kept[j][t] (added in ascending j, the new result last), whose copy `copy` then is:
+// a layer's last sublayer and the weighted sum over all layer results that follows it, in one pass.
 template <typename TY, typename TW, typename TA>
-__global__ void norm_residual_kernel(float* __restrict__ out, TA* __restrict__ copy, const float* __restrict__ base,
-                                     const TY* __restrict__ y, const TW* __restrict__ w, float eps, int H) {
+__global__ void norm_residual_kernel(float* out, TA* __restrict__ copy, const float* base,
+                                     const TY* __restrict__ y, const TW* __restrict__ w, float eps, int H,
+                                     float* __restrict__ mixed, const float* __restrict__ kept, size_t stride,
+                                     const TW* __restrict__ mix, int n) {
     __shared__ float red[16];
     const size_t off = (size_t)blockIdx.x * H;
     const TY* yr = y + off;
@@ -93,18 +98,27 @@ __global__ void norm_residual_kernel(float* __restrict__ out, TA* __restrict__ c
     ss = block_sum(ss, red);
     const float scale = 1.0f / sqrtf(ss / (float)H + eps);
     for (int i = threadIdx.x; i < H; i += blockDim.x) {
-        const float v = base[off + i] + (scale * to_f32<TY>(yr[i])) * to_f32<TW>(w[i]);
+        float v = base[off + i] + (scale * to_f32<TY>(yr[i])) * to_f32<TW>(w[i]);
         out[off + i] = v;
+        if (mixed) {
+            float s = 0.f;
+            for (int j = 0; j + 1 < n; ++j) s = fmaf(to_f32<TW>(mix[j]), kept[(size_t)j * stride + off + i], s);
+            v = fmaf(to_f32<TW>(mix[n - 1]), v, s);
+            mixed[off + i] = v;
+        }
         if (copy) copy[off + i] = from_f32<TA>(v);
     }
 }
 
 extern "C" int spy_norm_residual(float* out, void* copy, int copy_dtype, const float* base, const void* y, int y_dtype,
-                                 const void* w, int w_dtype, float eps, int T, int H, hipStream_t st) {
+                                 const void* w, int w_dtype, float eps, int T, int H, float* mixed, const float* kept,
+                                 long long stride, const void* mix, int n, hipStream_t st) {
     SPY_REQUIRE(T > 0 && H > 0, "spy_norm_residual: empty operand");
+    SPY_REQUIRE(!mixed || (kept && mix && n > 0 && stride >= (long long)T * H && out == kept + (size_t)(n - 1) * stride),
+                "spy_norm_residual: the mix needs the kept results, whose last one is this result, and their weights");
     const int threads = H >= 2048 ? 512 : (H >= 512 ? 256 : 64);
     SPY_DISPATCH(y_dtype, TY, SPY_DISPATCH(w_dtype, TW, SPY_DISPATCH(copy_dtype, TA, (norm_residual_kernel<TY, TW, TA><<<T, threads, 0, st>>>(
-        out, (TA*)copy, base, (const TY*)y, (const TW*)w, eps, H)))));
+        out, (TA*)copy, base, (const TY*)y, (const TW*)w, eps, H, mixed, kept, (size_t)stride, (const TW*)mix, n)))));
     SPY_CHECK_LAUNCH("spy_norm_residual");
     return 0;
 }

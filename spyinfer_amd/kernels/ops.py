@@ -888,9 +888,12 @@ def pair_embedding(ids: torch.Tensor, table: torch.Tensor, pair: Optional[torch.
 
 
 def norm_residual(base: torch.Tensor, y: torch.Tensor, weight: torch.Tensor, eps: float, out: Optional[torch.Tensor] = None,
-                  copy_dtype: Optional[torch.dtype] = None):
+                  copy_dtype: Optional[torch.dtype] = None, mix=None):
     """out = base + y / sqrt(mean(y^2) + eps) * weight, float32 (``out`` may be ``base``; a new tensor if None).
-    Returns (out, copy of out in ``copy_dtype`` or None)."""
+    Returns (out, copy of out in ``copy_dtype`` or None).
+
+    ``mix`` = (kept [layers, T, H] float32, n, a [n]): ``out`` must be ``kept[n - 1]``; the kernel also forms
+    sum_j a[j] * kept[j] over j < n (``depth_mix`` in the same pass) and returns (that sum, its copy) instead."""
     _dev(base, y, weight, out)
     _check(base.dtype == torch.float32 and base.dim() == 2, "norm_residual: the stream must be float32 [T, H]")
     T, H = base.shape
@@ -898,11 +901,21 @@ def norm_residual(base: torch.Tensor, y: torch.Tensor, weight: torch.Tensor, eps
     if out is None:
         out = torch.empty_like(base)
     _check(out.dtype == torch.float32 and tuple(out.shape) == (T, H), "norm_residual: out must be float32 [T, H]")
+    mixed = kept = a = None
+    n = 0
+    if mix is not None:
+        kept, n, a = mix
+        _dev(kept, a)
+        _check(kept.dtype == torch.float32 and kept.dim() == 3 and tuple(kept.shape[1:]) == (T, H) and 0 < n <= kept.shape[0]
+               and out.data_ptr() == kept[n - 1].data_ptr(), "norm_residual: the result must be the last of the n kept results [layers, T, H]")
+        _check(a.shape == (n,) and a.dtype == weight.dtype, "norm_residual: one mix weight per kept result, of the norm weight's dtype")
+        mixed = torch.empty_like(base)
     copy = _copy_of(out, copy_dtype)
     if T:
         hip().call("spy_norm_residual", _ptr(out), _ptr(copy), BF16 if copy is not None else F32, _ptr(base), _ptr(y), _code(y, "y"),
-                   _ptr(weight), _code(weight, "norm weight"), ctypes.c_float(eps), ctypes.c_int(T), ctypes.c_int(H), _Hip.stream())
-    return out, copy
+                   _ptr(weight), _code(weight, "norm weight"), ctypes.c_float(eps), ctypes.c_int(T), ctypes.c_int(H), _ptr(mixed),
+                   _ptr(kept), ctypes.c_longlong(T * H), _ptr(a), ctypes.c_int(n), _Hip.stream())
+    return (out if mixed is None else mixed), copy
 
 
 def depth_mix(kept: torch.Tensor, n: int, a: torch.Tensor, copy_dtype: Optional[torch.dtype] = None):
@@ -1044,7 +1057,7 @@ LATENT_MFMA = True          # False forces the plain kernel for bfloat16 too (te
 def latent_attention_mfma_ok(dtype, R: int, D: int) -> bool:
     """Whether the MFMA kernel takes latent rows of D values of which R are the values: bfloat16, 16-byte pieces, and
     sums of a row tile that fit a wave's registers."""
-    return LATENT_MFMA and dtype == torch.bfloat16 and D % 8 == 0 and R % 8 == 0 and D <= 640 and R <= 512
+    return LATENT_MFMA and dtype == torch.bfloat16 and D % 8 == 0 and R % 8 == 0 and D <= 576 and R <= 512
 
 
 def latent_key_parts(num_tiles: int, max_keys: int) -> int:

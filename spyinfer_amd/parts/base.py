@@ -51,8 +51,10 @@ class Norm(Part):
         the hidden state."""
         raise NotImplementedError
 
-    def add_normed(self, base: torch.Tensor, y: torch.Tensor, out: Optional[torch.Tensor] = None, copy_dtype=None):
-        """out = base + norm(y), float32, for blocks that norm a sublayer's output; (out, copy in ``copy_dtype`` or None)."""
+    def add_normed(self, base: torch.Tensor, y: torch.Tensor, out: Optional[torch.Tensor] = None, copy_dtype=None, mix=None):
+        """out = base + norm(y), float32, for blocks that norm a sublayer's output; (out, copy in ``copy_dtype`` or None).
+        ``mix`` = (kept layer results, n, weights): also the weighted sum of the n kept results, of which ``out`` is the
+        last, returned in place of ``out``."""
         raise NotImplementedError
 
     def foldable(self, out_dtype: torch.dtype):

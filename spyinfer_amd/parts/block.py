@@ -107,8 +107,13 @@ class DepthMix(Part):
         """Where this layer's result X_(index+1) is to be written."""
         return self.kept(batch, resid)[self.index + 1]
 
+    def operands(self, batch):
+        """(kept results, how many of them are mixed, their weights): what the kernel that writes this layer's result
+        needs to form the mix in the same pass (``Norm.add_normed``)."""
+        return batch.shared["depth_kept"], self.index + 2, self.weight
+
     def mix(self, batch):
-        """(the stream for the next layer, its copy in the activation dtype or None)."""
+        """(the stream for the next layer, its copy in the activation dtype or None), as a pass of its own."""
         return ops.depth_mix(batch.shared["depth_kept"], self.index + 2, self.weight, batch.act_dtype)
 
 
@@ -144,13 +149,12 @@ class OutputNormBlock(Block):
         x = stream_copy(batch, resid)
         y = self.mixer.forward(x, batch, cache, store)
         out = self.depth.result_slot(batch, resid) if self.depth is not None else resid
+        mix = self.depth.operands(batch) if self.depth is not None else None       # formed by the layer's last norm kernel
         last = self.ffn is None
-        out, copy = self.norm1.add_normed(resid, y, out, None if (last and self.depth is not None) else act)
+        out, copy = self.norm1.add_normed(resid, y, out, act, mix if last else None)
         if not last:
             x = stream_copy(batch, out, copy)
             f = self.ffn.forward(x, batch)
-            out, copy = self.norm2.add_normed(out, f, out, None if self.depth is not None else act)
-        if self.depth is not None:
-            out, copy = self.depth.mix(batch)
+            out, copy = self.norm2.add_normed(out, f, out, act, mix)
         stream_copy(batch, out, copy)
         return out, None

@@ -31,10 +31,14 @@ class RMSNorm(Norm):
     def add_norm(self, resid, delta, out_dtype, rows=None):
         return ops.add_rms_norm(resid, delta, self.weight, self.eps, out_dtype, rows)
 
-    def add_normed(self, base, y, out=None, copy_dtype=None):
+    def add_normed(self, base, y, out=None, copy_dtype=None, mix=None):
         """out = base + norm(y) in float32 (the norm on a sublayer's output; ``out`` may be ``base``); returns (out, its
-        copy in ``copy_dtype`` or None)."""
-        return ops.norm_residual(base, y, self.weight, self.eps, out, copy_dtype)
+        copy in ``copy_dtype`` or None).  ``mix`` = (kept results [layers, T, H], n, weights [n]) with ``out`` the n-th
+        kept result: the weighted sum of the n results is formed in the same pass and returned in place of ``out``."""
+        if mix is not None and mix[2].dtype != self.weight.dtype:
+            out, _ = ops.norm_residual(base, y, self.weight, self.eps, out, None)
+            return ops.depth_mix(mix[0], mix[1], mix[2], copy_dtype)
+        return ops.norm_residual(base, y, self.weight, self.eps, out, copy_dtype, mix)
 
     def foldable(self, out_dtype):
         if out_dtype == torch.bfloat16 and self.weight is not None and self.weight.dtype == torch.bfloat16:

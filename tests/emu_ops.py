@@ -122,13 +122,15 @@ class EmuOps:
                 last_token[int(slot_ids[e])] = ids[int(cu_q[e + 1]) - 1]
         return out, self._copy(out, copy_dtype)
 
-    def norm_residual(self, base, y, weight, eps, out=None, copy_dtype=None):
+    def norm_residual(self, base, y, weight, eps, out=None, copy_dtype=None, mix=None):
         yf = y.float()
         r = base + yf * torch.rsqrt((yf * yf).mean(-1, keepdim=True) + eps) * weight.float()
         if out is None:
             out = r
         else:
             out.copy_(r)
+        if mix is not None:
+            return self.depth_mix(mix[0], mix[1], mix[2], copy_dtype)
         return out, self._copy(out, copy_dtype)
 
     def depth_mix(self, kept, n, a, copy_dtype=None):

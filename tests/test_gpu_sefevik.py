@@ -66,6 +66,14 @@ def test_stream_kernels(dtype):
         close(copy, ref, torch.bfloat16, what="norm_residual copy")
     kept = torch.randn((6, T, H), generator=g)
     a = torch.randn((4,), generator=g).to(DT[dtype])
+    # the same sum formed by the kernel that writes the newest of the kept results
+    held = kept.clone().to(dev)
+    mixed, copy = ops.norm_residual(base.to(dev), y.to(dev), w.to(dev), eps, held[3], DT[dtype], (held, 4, a.to(dev)))
+    close(held[3], ref, torch.float32, what="norm_residual into a kept result")
+    want = sum(a[j].double() * kept[j].double() for j in range(3)) + a[3].double() * ref
+    close(mixed, want, torch.float32, what="norm_residual with the mix")
+    if copy is not None:
+        close(copy, want, torch.bfloat16, what="copy of the mix")
     out, _ = ops.depth_mix(kept.to(dev), 4, a.to(dev), DT[dtype])
     close(out, sum(a[j].double() * kept[j].double() for j in range(4)), torch.float32, what="depth_mix")
     z = (2 * torch.randn((T, H), generator=g)).to(DT[dtype])
