@@ -26,16 +26,14 @@ __global__ void pair_embedding_kernel(float* __restrict__ out, TA* __restrict__ 
     const TW* row = table + (size_t)id * H;
     const TW* prow = nullptr;
     if (pair) {
+        // everything is asked for whether or not it is needed, so that the loads go out together: the token before, the
+        // entry with its first row and slot, the slot's last token
+        const int pos = positions[t], e = token_entry[t], before = ids[t > 0 ? t - 1 : 0];
+        const int first = cu_q[e], slot = slot_ids[e];
+        const int held = (slot >= 0 && slot < num_slots) ? last_token[slot] : 0;
         int r = buckets;
-        if (positions[t] > 0) {
-            const int e = token_entry[t];
-            int prev;
-            if (t == cu_q[e]) {
-                const int slot = slot_ids[e];
-                prev = (slot >= 0 && slot < num_slots) ? last_token[slot] : 0;
-            } else {
-                prev = ids[t - 1];
-            }
+        if (pos > 0) {
+            const int prev = t == first ? held : before;
             long long h = ((long long)prev * mul_prev + (long long)id * mul_cur) % (long long)buckets;
             if (h < 0) h += buckets;
             r = (int)h;
@@ -85,7 +83,8 @@ extern "C" int spy_pair_embedding(float* out, void* copy, int copy_dtype, const 
 // With `mix` (n weights): out[t] is one of n kept layer results, kept[n - 1][t], and the kernel also writes
 // mixed[t] = sum over j < n of mix[j] * kept[j][t] (added in ascending j, the new result last), whose copy `copy` then is:
 // a layer's last sublayer and the weighted sum over all layer results that follows it, in one pass.
-template <typename TY, typename TW, typename TA>
+#define NR_PER 8      // values of a row that a thread keeps in registers between the two passes
+template <typename TY, typename TW, typename TA, bool REG>
 __global__ void norm_residual_kernel(float* out, TA* __restrict__ copy, const float* base,
                                      const TY* __restrict__ y, const TW* __restrict__ w, float eps, int H,
                                      float* __restrict__ mixed, const float* __restrict__ kept, size_t stride,
@@ -94,6 +93,45 @@ __global__ void norm_residual_kernel(float* out, TA* __restrict__ copy, const fl
     const size_t off = (size_t)blockIdx.x * H;
     const TY* yr = y + off;
     float ss = 0.f;
+    if (REG) {
+        // H <= NR_PER * blockDim.x: y is read once; what does not depend on the sum of squares (the stream's old values,
+        // the norm weight, the other kept results) is asked for before the block's sum, so that one memory round trip
+        // covers all of it
+        float yv[NR_PER], bv[NR_PER], wv[NR_PER], sv[NR_PER];
+#pragma unroll
+        for (int e = 0; e < NR_PER; ++e) {
+            const int i = threadIdx.x + e * blockDim.x;
+            yv[e] = i < H ? to_f32<TY>(yr[i]) : 0.f;
+            bv[e] = i < H ? base[off + i] : 0.f;
+            wv[e] = i < H ? to_f32<TW>(w[i]) : 0.f;
+            sv[e] = 0.f;
+            ss += yv[e] * yv[e];
+        }
+        if (mixed) {
+            for (int j = 0; j + 1 < n; ++j) {
+                const float a = to_f32<TW>(mix[j]);
+#pragma unroll
+                for (int e = 0; e < NR_PER; ++e) {
+                    const int i = threadIdx.x + e * blockDim.x;
+                    if (i < H) sv[e] = fmaf(a, kept[(size_t)j * stride + off + i], sv[e]);
+                }
+            }
+        }
+        ss = block_sum(ss, red);
+        const float scale = 1.0f / sqrtf(ss / (float)H + eps);
+        const float a_last = mixed ? to_f32<TW>(mix[n - 1]) : 0.f;
+#pragma unroll
+        for (int e = 0; e < NR_PER; ++e) {
+            const int i = threadIdx.x + e * blockDim.x;
+            if (i < H) {
+                float v = bv[e] + (scale * yv[e]) * wv[e];
+                out[off + i] = v;
+                if (mixed) { v = fmaf(a_last, v, sv[e]); mixed[off + i] = v; }
+                if (copy) copy[off + i] = from_f32<TA>(v);
+            }
+        }
+        return;
+    }
     for (int i = threadIdx.x; i < H; i += blockDim.x) { const float v = to_f32<TY>(yr[i]); ss += v * v; }
     ss = block_sum(ss, red);
     const float scale = 1.0f / sqrtf(ss / (float)H + eps);
@@ -117,8 +155,13 @@ extern "C" int spy_norm_residual(float* out, void* copy, int copy_dtype, const f
     SPY_REQUIRE(!mixed || (kept && mix && n > 0 && stride >= (long long)T * H && out == kept + (size_t)(n - 1) * stride),
                 "spy_norm_residual: the mix needs the kept results, whose last one is this result, and their weights");
     const int threads = H >= 2048 ? 512 : (H >= 512 ? 256 : 64);
-    SPY_DISPATCH(y_dtype, TY, SPY_DISPATCH(w_dtype, TW, SPY_DISPATCH(copy_dtype, TA, (norm_residual_kernel<TY, TW, TA><<<T, threads, 0, st>>>(
-        out, (TA*)copy, base, (const TY*)y, (const TW*)w, eps, H, mixed, kept, (size_t)stride, (const TW*)mix, n)))));
+    if (H <= NR_PER * threads) {
+        SPY_DISPATCH(y_dtype, TY, SPY_DISPATCH(w_dtype, TW, SPY_DISPATCH(copy_dtype, TA, (norm_residual_kernel<TY, TW, TA, true><<<T, threads, 0, st>>>(
+            out, (TA*)copy, base, (const TY*)y, (const TW*)w, eps, H, mixed, kept, (size_t)stride, (const TW*)mix, n)))));
+    } else {
+        SPY_DISPATCH(y_dtype, TY, SPY_DISPATCH(w_dtype, TW, SPY_DISPATCH(copy_dtype, TA, (norm_residual_kernel<TY, TW, TA, false><<<T, threads, 0, st>>>(
+            out, (TA*)copy, base, (const TY*)y, (const TW*)w, eps, H, mixed, kept, (size_t)stride, (const TW*)mix, n)))));
+    }
     SPY_CHECK_LAUNCH("spy_norm_residual");
     return 0;
 }

@@ -126,7 +126,7 @@ class LatentAttention(Mixer):
                                                              else "with a projection of its own was told to read another's cache"))
         nh, dn, dr, dv, r = self.heads, self.dim, self.rot_dim, self.vdim, self.kv_rank
         T = x.shape[0]
-        qd = ops.linear(x, self.w_in, tiled=self.w_in_tiled)
+        qd = ops.linear_few(x, self.w_in, self.w_in_tiled)
         nq = nh * (dn + dr)
         freq, mag, dims = self._frequencies()
         mfma = ("latent_tiles", nh) in batch.shared            # planned: the MFMA kernel takes these rows (bfloat16 queries)
@@ -159,4 +159,4 @@ class LatentAttention(Mixer):
                 ops.head_products(lat, nh * r, r, self.w_uv, v, nh * dv, dv, T)
             else:
                 ops.gemm_strided(lat, (r, nh * r, 1), self.w_uv, (dv * r, r, 1), v, (dv, nh * dv, 1), nh, T, dv, r)
-        return ops.linear(v, self.w_o, tiled=self.w_o_tiled)
+        return ops.linear_few(v, self.w_o, self.w_o_tiled)

@@ -79,4 +79,4 @@ class DenseMLP(FeedForward):
         return True
 
     def forward(self, x, batch):
-        return ops.linear(ops.linear_xielu(x, self.w_up, self.act, tiled=self.w_up_tiled), self.w_down, tiled=self.w_down_tiled)
+        return ops.linear_few(ops.linear_xielu(x, self.w_up, self.act, tiled=self.w_up_tiled), self.w_down, self.w_down_tiled)

@@ -78,7 +78,7 @@ class MinGRU(Mixer):
     def forward(self, x, batch, cache, store=True):
         if not store:
             raise ValueError("a recurrence cannot run on another layer's state without writing it")
-        zxg = ops.linear(x, self.w_zxg, tiled=self.w_zxg_tiled)
+        zxg = ops.linear_few(x, self.w_zxg, self.w_zxg_tiled)
         n, multi = batch.shared["scan_pieces"]
         y = ops.mingru(zxg, self.b_z, self.b_x, cache.state, batch.array("scan_pieces"), n, multi, batch.array("slot_ids"))
-        return ops.linear(y, self.w_o, tiled=self.w_o_tiled)
+        return ops.linear_few(y, self.w_o, self.w_o_tiled)
