@@ -239,13 +239,12 @@ typedef __attribute__((__vector_size__(8 * sizeof(short)))) short lbf16x8_t;
 typedef __attribute__((__vector_size__(4 * sizeof(float)))) float lf32x4_t;
 typedef __attribute__((__vector_size__(4 * sizeof(uint32_t)))) uint32_t lu32x4_t;
 
-#define LW 4          // waves (row tiles) per block
 #define LKPAD 8       // bf16 of padding per staged key row
 #define LVROW 40      // bf16 per row of the transposed values (32 keys + 8 of padding)
 
 // QS: most 32-wide steps of D; RT: most 16-wide tiles of R (both bound the registers)
-template <int QS, int RT, typename TW>
-__global__ __launch_bounds__(LW * 64) void latent_attention_mfma_kernel(
+template <int QS, int RT, int NW, typename TW>
+__global__ __launch_bounds__(NW * 64) void latent_attention_mfma_kernel(
     bf16_t* __restrict__ out, float* __restrict__ ws, const bf16_t* __restrict__ qa, const bf16_t* __restrict__ cache, int P,
     int num_pages, const int* __restrict__ cu_q, const int* __restrict__ pos0, const int* __restrict__ kv_len,
     const int* __restrict__ block_table, int max_blocks, const int* __restrict__ tile_entry, const int* __restrict__ tile_row0,
@@ -259,7 +258,7 @@ __global__ __launch_bounds__(LW * 64) void latent_attention_mfma_kernel(
     const int n_rows = (cu_q[e + 1] - q0) * H;
     const int r_lo = tile_row0[tile];
     if (r_lo >= n_rows) return;
-    const int r_hi = min(r_lo + 16 * LW, n_rows) - 1;
+    const int r_hi = min(r_lo + 16 * NW, n_rows) - 1;
     const int p0 = pos0[e], kvl = kv_len[e];
     const int p_lo = p0 + r_lo / H, p_hi = min(p0 + r_hi / H, kvl - 1);
     const int lo = window > 0 ? max(0, p_lo - window + 1) : 0;
@@ -298,7 +297,7 @@ __global__ __launch_bounds__(LW * 64) void latent_attention_mfma_kernel(
     // along d would all hit one bank), and a thread looks up one page per chunk.  The pieces of chunk c + 2 are asked for
     // (into registers) before chunk c is multiplied, and chunk c + 1 is written to the second LDS buffer before that: one
     // barrier per chunk, and no wave waits for memory while another has products to do.
-    constexpr int NP = (QS + 1) / 2;
+    constexpr int NP = (QS * 4 + NW * 2 - 1) / (NW * 2);             // 16-byte pieces of a key's row per thread
     const int sk = tid & 31, sd0 = (tid >> 5) * 8;
     const int buf_elems = 32 * krow + r_tiles * 16 * LVROW;
     lu32x4_t pf[NP];
@@ -311,7 +310,7 @@ __global__ __launch_bounds__(LW * 64) void latent_attention_mfma_kernel(
         }
 #pragma unroll
         for (int it = 0; it < NP; ++it) {
-            const int d8 = sd0 + 64 * it;
+            const int d8 = sd0 + 16 * NW * it;
             pf[it] = lu32x4_t{0u, 0u, 0u, 0u};
             if (src && d8 < D) pf[it] = *reinterpret_cast<const lu32x4_t*>(src + d8);
         }
@@ -321,7 +320,7 @@ __global__ __launch_bounds__(LW * 64) void latent_attention_mfma_kernel(
         bf16_t* vt = ks + 32 * krow;
 #pragma unroll
         for (int it = 0; it < NP; ++it) {
-            const int d8 = sd0 + 64 * it;
+            const int d8 = sd0 + 16 * NW * it;
             if (d8 < Dp) {
                 *reinterpret_cast<lu32x4_t*>(ks + sk * krow + d8) = pf[it];
                 if (d8 < r_tiles * 16) {
@@ -457,35 +456,38 @@ extern "C" long long spy_latent_attention_mfma_workspace(int T, int H, int R, in
     return splits > 1 ? (long long)T * H * splits * (R + 2) : 0;
 }
 
-// tiles: num_tiles records (entry, first row) of 64 rows each.  ws: float32, spy_latent_attention_mfma_workspace values.
+// tiles: num_tiles records (entry, first row) of tile_rows (64 or 128) rows each: a block of 4 or 8 waves.  ws: float32, spy_latent_attention_mfma_workspace values.
 extern "C" int spy_latent_attention_mfma(void* out, float* ws, const void* qa, const void* cache, int P, int num_pages,
                                          const int* cu_q, const int* pos0, const int* kv_len, const int* block_table,
                                          int max_blocks, const int* tile_entry, const int* tile_row0, int num_tiles,
                                          const void* sink, int sink_dtype, int T, int H, int R, int DR, float scale, int window,
-                                         int splits, hipStream_t st) {
+                                         int splits, int tile_rows, hipStream_t st) {
     const int D = R + DR;
     SPY_REQUIRE(T > 0 && H > 0 && R > 0 && DR >= 0 && P > 0 && num_pages > 0 && max_blocks > 0 && num_tiles > 0,
                 "spy_latent_attention_mfma: empty operand");
     SPY_REQUIRE(D % 8 == 0 && R % 8 == 0 && D <= 576 && R <= 512, "spy_latent_attention_mfma: rows of %d + %d values are not taken", R, DR);
+    SPY_REQUIRE(tile_rows == 64 || tile_rows == 128, "spy_latent_attention_mfma: tiles of %d rows (64 or 128)", tile_rows);
     SPY_REQUIRE(splits >= 1 && splits <= 64 && (splits == 1 || ws), "spy_latent_attention_mfma: %d parts (1..64, with a workspace)", splits);
     SPY_REQUIRE(((uintptr_t)qa % 16) == 0 && ((uintptr_t)cache % 16) == 0 && ((uintptr_t)out % 8) == 0, "spy_latent_attention_mfma: operands are not aligned");
     const int q_steps = (D + 31) / 32, r_tiles = (R + 15) / 16;
     const size_t lds = 2 * ((size_t)32 * (q_steps * 32 + LKPAD) + (size_t)r_tiles * 16 * LVROW) * sizeof(bf16_t);
     SPY_REQUIRE(lds <= 160 * 1024, "spy_latent_attention_mfma: two staged chunks of %d + %d values take %zu bytes of LDS", R, DR, lds);
     const dim3 grid(num_tiles, splits);
-#define SPY_LA_LAUNCH(QS, RT)                                                                                                   \
+#define SPY_LA_LAUNCH_W(QS, RT, NW)                                                                                             \
     SPY_DISPATCH(sink_dtype, TW, {                                                                                              \
-        auto kernel = latent_attention_mfma_kernel<QS, RT, TW>;                                                                 \
+        auto kernel = latent_attention_mfma_kernel<QS, RT, NW, TW>;                                                             \
         if (lds > 48 * 1024) {                                                                                                  \
             hipError_t e_ = hipFuncSetAttribute((const void*)kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);      \
             if (e_ != hipSuccess) return spy_fail("spy_latent_attention_mfma: %zu bytes of LDS refused: %s", lds, hipGetErrorString(e_)); \
         }                                                                                                                       \
-        kernel<<<grid, LW * 64, lds, st>>>((bf16_t*)out, ws, (const bf16_t*)qa, (const bf16_t*)cache, P, num_pages, cu_q, pos0, kv_len,        \
+        kernel<<<grid, NW * 64, lds, st>>>((bf16_t*)out, ws, (const bf16_t*)qa, (const bf16_t*)cache, P, num_pages, cu_q, pos0, kv_len, \
                                            block_table, max_blocks, tile_entry, tile_row0, (const TW*)sink, H, R, D, scale, window); \
     })
+#define SPY_LA_LAUNCH(QS, RT) if (tile_rows == 128) { SPY_LA_LAUNCH_W(QS, RT, 8); } else { SPY_LA_LAUNCH_W(QS, RT, 4); }
     if (q_steps <= 8 && r_tiles <= 8) { SPY_LA_LAUNCH(8, 8); }
     else if (q_steps <= 12 && r_tiles <= 16) { SPY_LA_LAUNCH(12, 16); }
     else { SPY_LA_LAUNCH(18, 32); }
+#undef SPY_LA_LAUNCH_W
 #undef SPY_LA_LAUNCH
     SPY_CHECK_LAUNCH("spy_latent_attention_mfma");
     if (splits > 1) {

@@ -1063,7 +1063,12 @@ def head_products(x: torch.Tensor, xt: int, xh: int, w: torch.Tensor, out: torch
 #: most rows of a step for which the per-head products of the latent attention run on ``head_products``; more rows take
 #: the library's batched product
 HEAD_PRODUCTS_MAX_ROWS = 128
-LATENT_TILE_ROWS = 64       # query rows, (token, head) pairs, of one block of the MFMA latent attention
+LATENT_TILE_ROWS = 64       # query rows, (token, head) pairs, of one block of the MFMA latent attention (4 waves)
+LATENT_TILE_ROWS_MANY = 128  # the same for steps with rows for every compute unit twice over (8 waves: a staged chunk of keys serves twice the rows)
+
+
+def latent_tile_rows(total_rows: int) -> int:
+    return LATENT_TILE_ROWS_MANY if total_rows >= LATENT_TILE_ROWS_MANY * 512 else LATENT_TILE_ROWS
 LATENT_MFMA = True          # False forces the plain kernel for bfloat16 too (tests flip it; nothing else does)
 
 
@@ -1096,8 +1101,9 @@ def latent_attention(qa: torch.Tensor, cache: torch.Tensor, page_size: int, meta
     _check(meta.block_table.shape == (meta.S, meta.max_blocks), "latent_attention: block table must be [S, max_blocks]")
     out = torch.empty((T, H, R), dtype=out_dtype, device=qa.device)
     if T and mfma:
-        # tiles: (entry [n], first row [n], n) of LATENT_TILE_ROWS rows each, planned on the host
-        tile_entry, tile_row0, n = tiles
+        # tiles: (entry [n], first row [n], n, rows of a tile) planned on the host
+        tile_entry, tile_row0, n = tiles[:3]
+        tile_rows = tiles[3] if len(tiles) > 3 else LATENT_TILE_ROWS
         _dev(tile_entry, tile_row0, meta.cu_q, meta.pos0)
         _check(n > 0 and tile_entry.shape == (n,) and tile_row0.shape == (n,), "latent_attention: the tiles' arrays do not fit their number")
         ws = None
@@ -1108,7 +1114,8 @@ def latent_attention(qa: torch.Tensor, cache: torch.Tensor, page_size: int, meta
                    ctypes.c_int(cache.shape[0]), _ptr(meta.cu_q), _ptr(meta.pos0), _ptr(meta.kv_len), _ptr(meta.block_table),
                    ctypes.c_int(meta.max_blocks), _ptr(tile_entry), _ptr(tile_row0), ctypes.c_int(n), _ptr(sink),
                    _code(sink, "sink") if sink is not None else F32, ctypes.c_int(T), ctypes.c_int(H), ctypes.c_int(R),
-                   ctypes.c_int(D - R), ctypes.c_float(scale), ctypes.c_int(int(window or 0)), ctypes.c_int(key_parts), _Hip.stream())
+                   ctypes.c_int(D - R), ctypes.c_float(scale), ctypes.c_int(int(window or 0)), ctypes.c_int(key_parts), ctypes.c_int(tile_rows),
+                   _Hip.stream())
         return out
     if T:
         hip().call("spy_latent_attention", _ptr(out), _code(out, "out"), _ptr(qa), _ptr(cache), _code(cache, "cache"),

@@ -96,7 +96,7 @@ class LatentAttention(Mixer):
         note = ("latent_tiles", self.heads)
         if note not in batch.shared:
             rows = batch.lens.astype(np.int64) * self.heads
-            size = ops.LATENT_TILE_ROWS
+            size = ops.latent_tile_rows(int(rows.sum()))
             counts = (rows + size - 1) // size
             entry = np.repeat(np.arange(batch.S, dtype=np.int64), counts)
             first = np.zeros(batch.S + 1, dtype=np.int64)
@@ -105,6 +105,7 @@ class LatentAttention(Mixer):
             batch.add_array("latent_tile_entry_%d" % self.heads, entry)
             batch.add_array("latent_tile_row0_%d" % self.heads, row0)
             batch.shared[note] = int(first[-1])
+            batch.shared[("latent_tile_rows", self.heads)] = size
         keys = batch.max_kv_len if self.window is None else min(batch.max_kv_len, self.window + batch.max_q_len - 1)
         parts = ops.latent_key_parts(batch.shared[note], keys)
         batch.shared[("latent_parts", self.heads, self.window)] = parts
@@ -147,7 +148,8 @@ class LatentAttention(Mixer):
         meta = attention_meta(batch, cache.group, nh)
         tiles, parts = None, 1
         if mfma:
-            tiles = (batch.array("latent_tile_entry_%d" % nh), batch.array("latent_tile_row0_%d" % nh), batch.shared[("latent_tiles", nh)])
+            tiles = (batch.array("latent_tile_entry_%d" % nh), batch.array("latent_tile_row0_%d" % nh), batch.shared[("latent_tiles", nh)],
+                     batch.shared[("latent_tile_rows", nh)])
             parts = batch.shared[("latent_parts", nh, self.window)]
         lat = ops.latent_attention(qa, cache.rows, cache.page_size, meta, self.sink, r, self.scale, self.window, x.dtype, tiles, parts)
         # the summed latents through the values' expansion: v[t, h, e] = sum_j lat[t, h, j] Wuv[h dv + e, j]

@@ -136,7 +136,9 @@ def test_mingru_scan_in_pieces_carries_the_state(dtype):
 @pytest.mark.parametrize("case", [dict(H=16, R=512, DR=64, P=16, window=300, entries=[(700, 1), (40, 1), (299, 1), (1500, 1)], parts=6),
                                   dict(H=16, R=512, DR=64, P=16, window=300, entries=[(0, 350), (811, 5), (64, 1)], parts=1),
                                   dict(H=5, R=96, DR=32, P=8, window=None, entries=[(0, 70), (130, 3), (257, 1)], parts=3),
-                                  dict(H=72, R=40, DR=8, P=32, window=33, entries=[(100, 1), (0, 45)], parts=2)])
+                                  dict(H=72, R=40, DR=8, P=32, window=33, entries=[(100, 1), (0, 45)], parts=2),
+                                  dict(H=16, R=512, DR=64, P=16, window=200, entries=[(0, 300), (500, 37), (64, 1)], parts=1, tile=128),
+                                  dict(H=6, R=64, DR=16, P=8, window=None, entries=[(0, 90), (130, 3)], parts=2, tile=128)])
 def test_latent_attention_on_mfma_equals_the_plain_kernel(case):
     """Rows of real sizes, a sink, a window that begins and ends inside pages and chunks, entries that are single tokens
     far into a request or portions from its start, keys in parts: against the float32 kernel on the same cache."""
@@ -165,8 +167,9 @@ def test_latent_attention_on_mfma_equals_the_plain_kernel(case):
     pos = np.concatenate([np.arange(p0, p0 + n) for p0, n in case["entries"]]).astype(np.int32)
     meta = ops.AttentionMeta(i32(cu, dev), i32([p0 for p0, _ in case["entries"]], dev), i32(kv, dev), torch.tensor(table, device=dev),
                              i32(ent, dev), i32(pos, dev), S, T, width, max(kv), max(lens))
-    counts = [-(-n * H // ops.LATENT_TILE_ROWS) for n in lens]
-    tiles = (i32(np.repeat(np.arange(S), counts), dev), i32(np.concatenate([np.arange(c) * ops.LATENT_TILE_ROWS for c in counts]), dev), sum(counts))
+    size = case.get("tile", ops.LATENT_TILE_ROWS)
+    counts = [-(-n * H // size) for n in lens]
+    tiles = (i32(np.repeat(np.arange(S), counts), dev), i32(np.concatenate([np.arange(c) * size for c in counts]), dev), sum(counts), size)
     ref = ops.latent_attention(qa, cache, P, meta, sink, R, 0.7, window, torch.float32)
     got = ops.latent_attention(qa.to(torch.bfloat16), cache, P, meta, sink, R, 0.7, window, torch.bfloat16, tiles, case["parts"])
     close(got, ref, torch.bfloat16, what="latent attention on MFMA")
