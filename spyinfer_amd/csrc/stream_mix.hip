@@ -7,13 +7,14 @@
 // ---------------------------------------------------------------------------------------------
 // out[t] = table[id[t]] + pair[row(t)], row = (prev * mul_prev + id * mul_cur) mod buckets, the last row (number
 // `buckets`) for a request's first token.  prev is the token before in the step, or for an entry's first token the one
-// that the request's state slot holds (`last_token`, written by the steps before).  copy (optional): the same values in
+// that the request's state slot holds (`last_token`, where the entry's last token is left for the next step).  copy
+// (optional): the same values in
 // the activation dtype, for the products that read the stream.
 template <typename TW, typename TA>
 __global__ void pair_embedding_kernel(float* __restrict__ out, TA* __restrict__ copy, const TW* __restrict__ table,
                                       const TW* __restrict__ pair, const int* __restrict__ ids, const int* __restrict__ positions,
                                       const int* __restrict__ token_entry, const int* __restrict__ cu_q,
-                                      const int* __restrict__ slot_ids, const int* __restrict__ last_token, int num_slots,
+                                      const int* __restrict__ slot_ids, int* last_token, int num_slots,
                                       int H, int V, int buckets, long long mul_prev, long long mul_cur) {
     const int t = blockIdx.x;
     const int id = ids[t];
@@ -26,19 +27,31 @@ __global__ void pair_embedding_kernel(float* __restrict__ out, TA* __restrict__ 
     const TW* row = table + (size_t)id * H;
     const TW* prow = nullptr;
     if (pair) {
-        // everything is asked for whether or not it is needed, so that the loads go out together: the token before, the
-        // entry with its first row and slot, the slot's last token
-        const int pos = positions[t], e = token_entry[t], before = ids[t > 0 ? t - 1 : 0];
-        const int first = cu_q[e], slot = slot_ids[e];
-        const int held = (slot >= 0 && slot < num_slots) ? last_token[slot] : 0;
-        int r = buckets;
-        if (pos > 0) {
-            const int prev = t == first ? held : before;
-            long long h = ((long long)prev * mul_prev + (long long)id * mul_cur) % (long long)buckets;
-            if (h < 0) h += buckets;
-            r = (int)h;
+        // One thread finds the row of the pair table and hands it to the block.  Everything it reads is asked for whether
+        // or not it is needed, so that the loads go out together: the token before, the entry with its first row and
+        // slot, the slot's last token.  The block of an entry's FIRST token is the only one that reads the slot, so it is
+        // also the one that leaves the entry's last token there: the same thread, after the barrier that its read's
+        // result had to reach first (no other block touches the slot in this step).
+        __shared__ int pair_row;
+        int e = 0, first = 0, slot = -1;
+        if (threadIdx.x == 0) {
+            const int pos = positions[t], before = ids[t > 0 ? t - 1 : 0];
+            e = token_entry[t];
+            first = cu_q[e];
+            slot = slot_ids[e];
+            const int held = (slot >= 0 && slot < num_slots) ? last_token[slot] : 0;
+            int r = buckets;
+            if (pos > 0) {
+                const int prev = t == first ? held : before;
+                long long h = ((long long)prev * mul_prev + (long long)id * mul_cur) % (long long)buckets;
+                if (h < 0) h += buckets;
+                r = (int)h;
+            }
+            pair_row = r;
         }
-        prow = pair + (size_t)r * H;
+        __syncthreads();
+        prow = pair + (size_t)pair_row * H;
+        if (threadIdx.x == 0 && t == first && slot >= 0 && slot < num_slots) last_token[slot] = ids[cu_q[e + 1] - 1];
     }
     for (int i = threadIdx.x; i < H; i += blockDim.x) {
         float v = to_f32<TW>(row[i]);
@@ -46,17 +59,6 @@ __global__ void pair_embedding_kernel(float* __restrict__ out, TA* __restrict__ 
         o[i] = v;
         if (c) c[i] = from_f32<TA>(v);
     }
-}
-
-// last_token[slot of entry e] = the entry's last token of this step (after every block above has read the old value:
-// it is a launch of its own)
-__global__ void keep_last_token_kernel(int* __restrict__ last_token, const int* __restrict__ ids, const int* __restrict__ cu_q,
-                                       const int* __restrict__ slot_ids, int S, int num_slots) {
-    const int e = blockIdx.x * blockDim.x + threadIdx.x;
-    if (e >= S) return;
-    const int slot = slot_ids[e];
-    const int n = cu_q[e + 1];
-    if (slot >= 0 && slot < num_slots && n > cu_q[e]) last_token[slot] = ids[n - 1];
 }
 
 extern "C" int spy_pair_embedding(float* out, void* copy, int copy_dtype, const void* table, const void* pair, int table_dtype,
@@ -70,10 +72,6 @@ extern "C" int spy_pair_embedding(float* out, void* copy, int copy_dtype, const 
         out, (TA*)copy, (const TW*)table, (const TW*)pair, ids, positions, token_entry, cu_q, slot_ids, last_token, num_slots, H, V,
         buckets, mul_prev, mul_cur))));
     SPY_CHECK_LAUNCH("spy_pair_embedding");
-    if (pair) {
-        keep_last_token_kernel<<<(S + 63) / 64, 64, 0, st>>>(last_token, ids, cu_q, slot_ids, S, num_slots);
-        SPY_CHECK_LAUNCH("spy_pair_embedding (last tokens)");
-    }
     return 0;
 }
 
