@@ -130,14 +130,18 @@ __global__ void norm_residual_kernel(float* out, TA* __restrict__ copy, const fl
         }
         return;
     }
+    // Few rows: gridDim.y blocks share a row.  Each forms the whole row's sum of squares (the row is a few kilobytes, from
+    // L2) and writes its slice of the outputs, so that a step of a handful of tokens still has blocks for many units.
     for (int i = threadIdx.x; i < H; i += blockDim.x) { const float v = to_f32<TY>(yr[i]); ss += v * v; }
     ss = block_sum(ss, red);
     const float scale = 1.0f / sqrtf(ss / (float)H + eps);
-    for (int i = threadIdx.x; i < H; i += blockDim.x) {
+    const int lo = (int)((long long)H * blockIdx.y / gridDim.y), hi = (int)((long long)H * (blockIdx.y + 1) / gridDim.y);
+    for (int i = lo + threadIdx.x; i < hi; i += blockDim.x) {
         float v = base[off + i] + (scale * to_f32<TY>(yr[i])) * to_f32<TW>(w[i]);
         out[off + i] = v;
         if (mixed) {
             float s = 0.f;
+#pragma unroll 4
             for (int j = 0; j + 1 < n; ++j) s = fmaf(to_f32<TW>(mix[j]), kept[(size_t)j * stride + off + i], s);
             v = fmaf(to_f32<TW>(mix[n - 1]), v, s);
             mixed[off + i] = v;
@@ -153,7 +157,13 @@ extern "C" int spy_norm_residual(float* out, void* copy, int copy_dtype, const f
     SPY_REQUIRE(!mixed || (kept && mix && n > 0 && stride >= (long long)T * H && out == kept + (size_t)(n - 1) * stride),
                 "spy_norm_residual: the mix needs the kept results, whose last one is this result, and their weights");
     const int threads = H >= 2048 ? 512 : (H >= 512 ? 256 : 64);
-    if (H <= NR_PER * threads) {
+    if (T <= 128 && H >= 1024) {
+        // rows for fewer blocks than the device has units: several blocks per row
+        const int per_row = T <= 32 ? 8 : (T <= 64 ? 4 : 2);
+        const dim3 grid(T, per_row);
+        SPY_DISPATCH(y_dtype, TY, SPY_DISPATCH(w_dtype, TW, SPY_DISPATCH(copy_dtype, TA, (norm_residual_kernel<TY, TW, TA, false><<<grid, 256, 0, st>>>(
+            out, (TA*)copy, base, (const TY*)y, (const TW*)w, eps, H, mixed, kept, (size_t)stride, (const TW*)mix, n)))));
+    } else if (H <= NR_PER * threads) {
         SPY_DISPATCH(y_dtype, TY, SPY_DISPATCH(w_dtype, TW, SPY_DISPATCH(copy_dtype, TA, (norm_residual_kernel<TY, TW, TA, true><<<T, threads, 0, st>>>(
             out, (TA*)copy, base, (const TY*)y, (const TW*)w, eps, H, mixed, kept, (size_t)stride, (const TW*)mix, n)))));
     } else {

@@ -52,11 +52,13 @@ def test_pair_embedding_keeps_the_previous_token_in_the_slot(dtype):
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
-def test_stream_kernels(dtype):
+@pytest.mark.parametrize("T,H", [(13, 50), (5, 2048), (70, 1100), (200, 4096), (3, 5000)])
+def test_stream_kernels(dtype, T, H):
+    """Rows whose values a thread keeps in registers, rows shared by several blocks (few rows), and the plain loop."""
     from spyinfer_amd.kernels import ops
     dev = require_gpu()
     g = torch.Generator().manual_seed(2)
-    T, H, eps = 13, 50, 1e-5
+    eps = 1e-5
     base, y = torch.randn((T, H), generator=g), (3 * torch.randn((T, H), generator=g)).to(DT[dtype])
     w = (1 + 0.2 * torch.randn((H,), generator=g)).to(DT[dtype])
     out, copy = ops.norm_residual(base.to(dev), y.to(dev), w.to(dev), eps, None, DT[dtype])
