@@ -86,7 +86,7 @@ def main(argv=None) -> int:
     if args.random_prompts:
         import torch
         g = torch.Generator().manual_seed(args.seed)
-        vocab = engine.model.config.vocab_size
+        vocab = engine.model.vocab_size
         prompts += [torch.randint(0, vocab, (n,), generator=g).tolist() for n in parse_ids(args.random_prompts)]
     if prompts:
         ids = [engine.add_request(p, params) for p in prompts]

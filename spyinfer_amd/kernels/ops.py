@@ -326,13 +326,14 @@ def linear(x: torch.Tensor, w: torch.Tensor, out_dtype: Optional[torch.dtype] = 
 DECODE_ROWS_PLAIN = 64
 
 
-def linear_few(x: torch.Tensor, w: torch.Tensor, tiled: Optional[torch.Tensor] = None, out_dtype: Optional[torch.dtype] = None) -> torch.Tensor:
+def linear_few(x: torch.Tensor, w: torch.Tensor, tiled: Optional[torch.Tensor] = None, out_dtype: Optional[torch.dtype] = None,
+               out: Optional[torch.Tensor] = None) -> torch.Tensor:
     """``linear`` for parts that do not fold norms into their products: up to DECODE_ROWS_PLAIN bfloat16 rows go to the
     decode products (which stream the tiled matrix once and beat the library there: 18.7 against 20.3 us for 6144 x 4096 at
     32 rows, 10.5 against 20.6 for 4096 x 4096), everything else to ``linear``."""
     if tiled is not None and x.dtype == torch.bfloat16 and x.dim() == 2 and 0 < x.shape[0] <= DECODE_ROWS_PLAIN and x.is_contiguous():
-        return decode_linear(x, tiled, out_dtype or torch.bfloat16)
-    return linear(x, w, out_dtype, tiled=tiled)
+        return decode_linear(x, tiled, out_dtype or torch.bfloat16, out)
+    return linear(x, w, out_dtype, tiled=tiled, out=out)
 
 
 def linear_swiglu(x: torch.Tensor, w_gate_up: torch.Tensor, tiled: Optional[torch.Tensor] = None) -> torch.Tensor:

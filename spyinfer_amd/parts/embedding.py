@@ -80,6 +80,8 @@ class LMHead(Part):
         """float32 logits [rows, vocab]; written into ``out`` if the caller brings a tensor of that shape."""
         if isinstance(normed, ops.ScaledInput):
             return ops.decode_linear(normed, self.weight_tiled, torch.float32, out)
+        if normed.shape[0] <= self.fold_rows:
+            return ops.linear_few(normed, self.weight, self.weight_tiled, torch.float32, out)      # the decode products, without a folded norm
         return ops.linear(normed, self.weight, torch.float32, tiled=self.weight_tiled, out=out)
 
 

@@ -287,3 +287,13 @@ def test_trace_run_as_a_program(folders, tmp_path):
                        capture_output=True, text=True, timeout=600)
     assert r.returncode == 0, r.stderr[-2000:]
     rc.compare(rc.collect(str(tmp_path), steps, 61), sc.plain_logits(folder, requests), what="trace_run", **TOL["float32"])
+
+
+def test_command_line_generates(folders):
+    require_gpu()
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    r = subprocess.run([sys.executable, "-m", "spyinfer_amd", "-m", folders["a"], "--dtype", "float32", "--random-prompts", "5,9",
+                        "--max-new-tokens", "6", "--max-model-len", "64", "--num-kvcache-blocks", "16", "--max-num-seqs", "4"],
+                       cwd=root, capture_output=True, text=True, timeout=600)
+    assert r.returncode == 0, r.stderr[-2000:]
+    assert r.stdout.strip(), "the command line printed no tokens"
