@@ -218,8 +218,30 @@ __global__ void xielu_kernel(TA* __restrict__ out, const TA* __restrict__ in, co
         out[i] = from_f32<TA>(xielu_f(to_f32<TA>(in[i]), ap, aq));
 }
 
+// the same, 8 bfloat16 values per thread and step with 16-byte loads and stores (count % 8 == 0, aligned)
+template <typename TW>
+__global__ void xielu_bf16x8_kernel(bf16_t* __restrict__ out, const bf16_t* __restrict__ in, const TW* __restrict__ pq, size_t count8) {
+    typedef __attribute__((__vector_size__(4 * sizeof(uint32_t)))) uint32_t u32x4_t;
+    const float ap = softplus_f(to_f32<TW>(pq[0])), aq = 0.5f + softplus_f(to_f32<TW>(pq[1]));
+    for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < count8; i += (size_t)gridDim.x * blockDim.x) {
+        const u32x4_t v = __builtin_nontemporal_load(reinterpret_cast<const u32x4_t*>(in) + i);
+        u32x4_t y;
+#pragma unroll
+        for (int e = 0; e < 4; ++e)
+            y[e] = pack_bf16x2(xielu_f(__uint_as_float(v[e] << 16), ap, aq), xielu_f(__uint_as_float(v[e] & 0xffff0000u), ap, aq));
+        reinterpret_cast<u32x4_t*>(out)[i] = y;
+    }
+}
+
 extern "C" int spy_xielu(void* out, const void* in, int dtype, const void* pq, int pq_dtype, long long count, hipStream_t st) {
     SPY_REQUIRE(count > 0, "spy_xielu: empty operand");
+    if (dtype == SPY_BF16 && count % 8 == 0 && ((uintptr_t)in % 16) == 0 && ((uintptr_t)out % 16) == 0) {
+        long long blocks = (count / 8 + 255) / 256;
+        if (blocks > 16384) blocks = 16384;
+        SPY_DISPATCH(pq_dtype, TW, (xielu_bf16x8_kernel<TW><<<(unsigned)blocks, 256, 0, st>>>((bf16_t*)out, (const bf16_t*)in, (const TW*)pq, (size_t)(count / 8))));
+        SPY_CHECK_LAUNCH("spy_xielu");
+        return 0;
+    }
     long long blocks = (count + 255) / 256;
     if (blocks > 8192) blocks = 8192;
     SPY_DISPATCH(dtype, TA, SPY_DISPATCH(pq_dtype, TW, (xielu_kernel<TA, TW><<<(unsigned)blocks, 256, 0, st>>>(

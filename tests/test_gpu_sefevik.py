@@ -85,14 +85,15 @@ def test_stream_kernels(dtype, T, H):
         close(got, plain.xielu(z.double(), float(t[0]), float(t[1])), DT[dtype], what="xielu %r" % (pq,))
 
 
+@pytest.mark.parametrize("W", [70, 33, 512])
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
-def test_mingru_scan_in_pieces_carries_the_state(dtype):
+def test_mingru_scan_in_pieces_carries_the_state(dtype, W):
     from spyinfer_amd.engine.batch import StepBatch  # noqa: F401  (the pieces are planned as the part plans them)
     from spyinfer_amd.kernels import ops
     from spyinfer_amd.parts import recurrent
     dev = require_gpu()
     g = torch.Generator().manual_seed(3)
-    W, lens = 70, [150, 1, 33]
+    lens = [150, 1, 33]
     zxg = torch.randn((sum(lens) * 2, 3 * W), generator=g).to(DT[dtype])
     bz, bx = torch.randn((W,), generator=g).to(DT[dtype]), torch.randn((W,), generator=g).to(DT[dtype])
     state = torch.zeros((5, W), dtype=torch.float32, device=dev)
