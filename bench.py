@@ -21,6 +21,7 @@ Other workloads, each again one JSON line:
 
     python bench.py --shape 14b --serve 64                 # Qwen3-14B shape: 64 requests at once until all have ended
     python bench.py --shape 32b --batch 64 --prompt-len 4096 --context 4608 --points "" --steps 32 --warmup 4   # long keys at the 32B shape
+    python bench.py --design sefevik [--design-sizes 1024,2048,4096] [--layers 8]   # Sefevik beside Qwen3 at equal size
 """
 import argparse
 import json
@@ -54,7 +55,7 @@ def sefevik_shape(width: int, layers: int, vocab: int, window: int = 1024) -> di
     dims, a latent of 512, a feed-forward of three times the width; of every four layers one latent attention with its
     own rows, two recurrences and one latent attention that reads the first one's rows."""
     heads = max(1, width // 128)
-    rot = dict(base=10000.0, dims=64, scaling=dict(factor=4.0, original=4096, fast=32.0, slow=1.0))
+    rot = dict(base=10000.0, dims=64, scaling=dict(factor=8.0, original=4096, fast=16.0, slow=2.0))
     att = dict(heads=heads, dim=128, rot_dim=64, vdim=128, kv_rank=512, scale=192 ** -0.5, mask=dict(size=window), rot=rot)
     out = []
     for i in range(layers):
@@ -65,8 +66,8 @@ def sefevik_shape(width: int, layers: int, vocab: int, window: int = 1024) -> di
             out.append(dict(type="latent_attention", mixer=dict(att, kv_from=i - 3), mlp=dict(kind="dense", ff=3 * width)))
         else:
             out.append(dict(type="mingru", mixer=dict(width=width), mlp=dict(kind="dense", ff=3 * width)))
-    return dict(architecture="Sefevik", vocab=vocab, width=width, norm=dict(eps=1e-5),
-                embedding=dict(bigram=dict(buckets=65521, mul_prev=31, mul_cur=7)), layers=out)
+    return dict(architecture="Sefevik", vocab=vocab, width=width, norm=dict(eps=1e-6),
+                embedding=dict(bigram=dict(buckets=65521, mul_prev=37, mul_cur=11)), layers=out)
 
 
 def design_compare(args) -> int:

@@ -40,22 +40,22 @@ SEF_A = dict(architecture="Sefevik", vocab=97, width=48, norm=dict(eps=3e-6),
 
 #: values that may happen to be equal or 1 elsewhere: one head, a window of one and of two tokens, equal sizes, a
 #: recurrence first, no pair table
-SEF_B = dict(architecture="Sefevik", vocab=61, width=32, norm=dict(eps=1e-5),
+SEF_B = dict(architecture="Sefevik", vocab=61, width=32, norm=dict(eps=2e-5),
              layers=[_layer("mingru", dict(width=32), ff=32),
                      _layer("latent_attention", _latent(1, 8, 8, 8, 8, 1.0, window=1), ff=40),
                      _layer("latent_attention", _latent(4, 8, 8, 8, 16, 0.5, window=2))])
 
 #: sizes that the products' tiled kernels take in bfloat16 (inner sizes in multiples of 128, outer ones of 16)
-SEF_C = dict(architecture="Sefevik", vocab=400, width=128, norm=dict(eps=1e-5),
-             embedding=dict(bigram=dict(buckets=211, mul_prev=31, mul_cur=3)),
-             layers=[_layer("latent_attention", _latent(4, 32, 16, 32, 112, 0.15, window=24, scaling=dict(factor=4.0, original=32, fast=8.0, slow=1.0)), ff=256),
+SEF_C = dict(architecture="Sefevik", vocab=400, width=128, norm=dict(eps=4e-6),
+             embedding=dict(bigram=dict(buckets=211, mul_prev=29, mul_cur=3)),
+             layers=[_layer("latent_attention", _latent(4, 32, 16, 32, 112, 0.15, window=24, scaling=dict(factor=3.0, original=32, fast=8.0, slow=1.5)), ff=256),
                      _layer("mingru", dict(width=128), ff=128),
                      _layer("latent_attention", _latent(4, 16, 16, 48, 112, 0.2, window=70, kv_from=0,
-                                                        scaling=dict(factor=4.0, original=32, fast=8.0, slow=1.0)), ff=256)])
+                                                        scaling=dict(factor=3.0, original=32, fast=8.0, slow=1.5)), ff=256)])
 
 #: one attention layer that sees everything: far keys
 SEF_FAR = dict(architecture="Sefevik", vocab=83, width=40, norm=dict(eps=1e-6),
-               embedding=dict(bigram=dict(buckets=29, mul_prev=3, mul_cur=7)),
+               embedding=dict(bigram=dict(buckets=29, mul_prev=3, mul_cur=13)),
                layers=[_layer("latent_attention", _latent(3, 12, 8, 10, 24, 0.35, base=100000.0), ff=48)])
 
 INIT = dict(matrix_std=0.12, norm_std=0.2, bias_std=0.7)
