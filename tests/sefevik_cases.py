@@ -83,6 +83,16 @@ def sharpen(factor=6.0):
     return tweak
 
 
+def heavy_sinks(value=3.0):
+    """Sinks that take most of every softmax's weight: a sink left out, counted twice or scaled changes every attention
+    output by a large factor."""
+    def tweak(tensors):
+        for name in tensors:
+            if name.endswith(".mix.sink"):
+                tensors[name] = (tensors[name].float() * 0.3 + value).to(tensors[name].dtype)
+    return tweak
+
+
 def plain_logits(folder, requests):
     plain = PlainSefevik.from_folder(folder)
     return {rid: plain.forward(toks) for rid, toks in requests.items()}

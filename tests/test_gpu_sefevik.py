@@ -178,6 +178,49 @@ def test_latent_attention_on_mfma_equals_the_plain_kernel(case):
     close(got, ref, torch.bfloat16, what="latent attention on MFMA")
 
 
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("dims,scaling", [(8, None), (6, dict(factor=8.0, original=64, fast=16.0, slow=2.0)), (0, None)])
+def test_latent_prepare_norms_rotates_and_stores(dtype, dims, scaling):
+    """The latent's norm, the rotation (all of the rotated part or its first dims, with and without scaled frequencies,
+    or none) of the shared key part and of every head's query part, and the store into the tokens' page rows."""
+    from spyinfer_amd.kernels import ops
+    from spyinfer_amd.parts import RotaryEmbedding
+    dev = require_gpu()
+    g = torch.Generator().manual_seed(7)
+    T, H, DN, DR, R, P, eps = 11, 3, 6, 8, 20, 4, 1e-5
+    ld = H * (DN + DR) + R + DR
+    qd = torch.randn((T, ld), generator=g).to(DT[dtype])
+    w = (1 + 0.3 * torch.randn((R,), generator=g)).to(DT[dtype])
+    pos = torch.tensor([0, 1, 2, 3, 4, 700, 701, 702, 9000, 9001, 33], dtype=torch.int32)
+    slots = torch.randperm(6 * P, generator=g)[:T].to(torch.int32)
+    cache = torch.full((6, P, R + DR), float("nan"), dtype=DT[dtype], device=dev)
+    freq = mag = None
+    if dims:
+        rot = RotaryEmbedding(DR, 5000.0, dims, scaling)
+        rot.prepare(dev, 0)
+        freq, mag, _ = rot.frequencies()
+    x = qd.to(dev)
+    qa = ops.latent_prepare(x, x[:, H * (DN + DR):], cache, slots.to(dev), w.to(dev), eps, freq, mag or 1.0, dims, pos.to(dev), H, DN, DR, R,
+                            DT[dtype])
+    d = qd.double()[:, H * (DN + DR):]
+    c_ref = plain.rms_norm(d[:, :R], w.double(), eps)
+    q_rot = qd.double()[:, :H * (DN + DR)].view(T, H, DN + DR)[:, :, DN:]
+    kr_ref = d[:, R:]
+    if dims:
+        f, m = plain.yarn_frequencies(dims, 5000.0, scaling)
+        kr_ref = plain.rotate_half(kr_ref, pos, f, m, dims)
+        q_rot = plain.rotate_half(q_rot.transpose(0, 1), pos, f, m, dims).transpose(0, 1)
+    rows = cache.view(-1, R + DR)[slots.long().to(dev)]
+    # angles are position * frequency in float32: at position 9000 that alone is 1e-3 of a turn's sine
+    tol = torch.float32 if dtype == "float32" else torch.bfloat16
+    close(rows[:, :R], c_ref, tol, what="latent")
+    close(rows[:, R:], kr_ref, tol, scale=40.0 if dtype == "float32" else 1.0, what="rotated key part")
+    close(qa[:, :, R:], q_rot, tol, scale=40.0 if dtype == "float32" else 1.0, what="rotated query parts")
+    untouched = torch.ones(6 * P, dtype=torch.bool)
+    untouched[slots.long()] = False
+    assert torch.isnan(cache.view(-1, R + DR)[untouched.to(dev)]).all(), "a row of another token was written"
+
+
 @pytest.mark.parametrize("T,H,N,K,out_dtype", [(1, 16, 512, 128, torch.bfloat16), (37, 3, 40, 72, torch.float32), (128, 8, 128, 512, torch.bfloat16)])
 def test_head_products(T, H, N, K, out_dtype):
     from spyinfer_amd.kernels import ops
@@ -195,6 +238,7 @@ def test_head_products(T, H, N, K, out_dtype):
 
 # ---- whole models under every schedule ------------------------------------------------------------
 MODELS = {"a": (sc.SEF_A, 3, None), "b": (sc.SEF_B, 4, None), "c": (sc.SEF_C, 6, None), "a_sharp": (sc.SEF_A, 5, sc.sharpen()),
+          "c_sink": (sc.SEF_C, 9, sc.heavy_sinks()),
           "far_sharp": (sc.SEF_FAR, 8, sc.sharpen(8.0))}
 
 
@@ -204,7 +248,7 @@ def folders(tmp_path_factory):
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
-@pytest.mark.parametrize("name", ["a", "b", "c", "a_sharp"])
+@pytest.mark.parametrize("name", ["a", "b", "c", "a_sharp", "c_sink"])
 @pytest.mark.parametrize("mode", ["whole", "bulk_tail", "portions", "mixed"])
 def test_schedules_equal_the_plain_implementation(folders, name, mode, dtype, tmp_path):
     require_gpu()
@@ -212,7 +256,7 @@ def test_schedules_equal_the_plain_implementation(folders, name, mode, dtype, tm
     requests = rc.random_requests(sc.vocab_of(folder), [41, 1, 2, 130, 23, 30, 52, 38, 75], 7)
     steps = {"whole": rc.whole, "bulk_tail": lambda r: rc.bulk_tail(r, 40), "portions": rc.portions, "mixed": rc.mixed}[mode](requests)
     rc.run_replay_inprocess(folder, dtype, str(tmp_path), steps, rc.max_live_tokens(steps),
-                            ["--kvcache-block-size", "8" if name != "c" else "16", "--poison-cache"])
+                            ["--kvcache-block-size", "8" if not name.startswith("c") else "16", "--poison-cache"])
     rc.compare(rc.collect(str(tmp_path), steps, sc.vocab_of(folder)), sc.plain_logits(folder, requests),
                what="%s/%s/%s" % (name, mode, dtype), **TOL[dtype])
 

@@ -17,7 +17,8 @@ TOL = dict(atol=2e-4, rtol=2e-4)
 @pytest.fixture(scope="module")
 def folders(tmp_path_factory):
     return {name: sc.write_model(str(tmp_path_factory.mktemp("sef_" + name)), cfg, seed, tweak)
-            for name, cfg, seed, tweak in (("a", sc.SEF_A, 3, None), ("b", sc.SEF_B, 4, None), ("a_sharp", sc.SEF_A, 5, sc.sharpen()))}
+            for name, cfg, seed, tweak in (("a", sc.SEF_A, 3, None), ("b", sc.SEF_B, 4, None), ("a_sharp", sc.SEF_A, 5, sc.sharpen()),
+                                        ("a_sink", sc.SEF_A, 9, sc.heavy_sinks()))}
 
 
 def test_configuration_is_read_by_name_and_checked():
@@ -49,7 +50,7 @@ def test_rows_are_kept_for_the_largest_window_that_reads_them():
     assert [(c.layer, c.cache, c.store) for c in model.schedule][2] == (2, 0, False)
 
 
-@pytest.mark.parametrize("name", ["a", "b", "a_sharp"])
+@pytest.mark.parametrize("name", ["a", "b", "a_sharp", "a_sink"])
 @pytest.mark.parametrize("mode", ["whole", "bulk_tail", "portions", "mixed"])
 def test_schedules_equal_the_plain_implementation(folders, name, mode, tmp_path, emu_ops):
     folder = folders[name]
