@@ -130,7 +130,9 @@ class LatentAttention(Mixer):
         qd = ops.linear_few(x, self.w_in, self.w_in_tiled)
         nq = nh * (dn + dr)
         freq, mag, dims = self._frequencies()
-        mfma = ("latent_tiles", nh) in batch.shared            # planned: the MFMA kernel takes these rows (bfloat16 queries)
+        # the MFMA kernel takes THIS layer's rows (another layer with as many heads may have planned tiles that this one
+        # cannot use): bfloat16 queries then, float32 ones for the plain kernel
+        mfma = ops.latent_attention_mfma_ok(batch.act_dtype, r, r + dr) and ("latent_parts", nh, self.window) in batch.shared
         qa = ops.latent_prepare(qd, qd[:, nq:] if store else None, cache.rows if store else None,
                                 batch.slot_mapping(cache.group) if store else None, self.c_norm, self.norm_eps, freq, mag, dims,
                                 batch.positions, nh, dn, dr, r, torch.bfloat16 if mfma else torch.float32)
