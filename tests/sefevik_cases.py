@@ -58,6 +58,16 @@ SEF_FAR = dict(architecture="Sefevik", vocab=83, width=40, norm=dict(eps=1e-6),
                embedding=dict(bigram=dict(buckets=29, mul_prev=3, mul_cur=13)),
                layers=[_layer("latent_attention", _latent(3, 12, 8, 10, 24, 0.35, base=100000.0), ff=48)])
 
+#: windows of hundreds of tokens over long requests, a reader with a shorter window than the rows' owner, rows of the
+#: width that the MFMA attention takes in its largest form's neighbourhood
+SEF_LONG = dict(architecture="Sefevik", vocab=211, width=64, norm=dict(eps=1e-6),
+                embedding=dict(bigram=dict(buckets=97, mul_prev=17, mul_cur=5)),
+                layers=[_layer("latent_attention", _latent(4, 16, 16, 16, 160, 0.3, window=333, base=50000.0,
+                                                           scaling=dict(factor=6.0, original=512, fast=24.0, slow=2.0)), ff=96),
+                        _layer("mingru", dict(width=48), ff=64),
+                        _layer("latent_attention", _latent(2, 8, 16, 24, 160, 0.4, window=150, kv_from=0, base=50000.0,
+                                                           scaling=dict(factor=6.0, original=512, fast=24.0, slow=2.0)))])
+
 INIT = dict(matrix_std=0.12, norm_std=0.2, bias_std=0.7)
 
 

@@ -238,7 +238,7 @@ def test_head_products(T, H, N, K, out_dtype):
 
 # ---- whole models under every schedule ------------------------------------------------------------
 MODELS = {"a": (sc.SEF_A, 3, None), "b": (sc.SEF_B, 4, None), "c": (sc.SEF_C, 6, None), "a_sharp": (sc.SEF_A, 5, sc.sharpen()),
-          "c_sink": (sc.SEF_C, 9, sc.heavy_sinks()),
+          "c_sink": (sc.SEF_C, 9, sc.heavy_sinks()), "long_sharp": (sc.SEF_LONG, 10, sc.sharpen(4.0)),
           "far_sharp": (sc.SEF_FAR, 8, sc.sharpen(8.0))}
 
 
@@ -271,6 +271,21 @@ def test_far_keys_among_hundreds(folders, mode, tmp_path):
     steps = {"whole": rc.whole, "bulk_tail": lambda r: rc.bulk_tail(r, 50), "portions": lambda r: rc.portions(r, (100, 3, 2, 257, 64, 1))}[mode](requests)
     rc.run_replay_inprocess(folder, "float32", str(tmp_path), steps, rc.max_live_tokens(steps), ["--poison-cache"])
     rc.compare(rc.collect(str(tmp_path), steps, sc.vocab_of(folder)), sc.plain_logits(folder, requests), what="far/" + mode, **TOL["float32"])
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("mode", ["whole", "bulk_tail", "portions", "mixed"])
+def test_long_requests_under_windows_of_hundreds(folders, mode, dtype, tmp_path):
+    """Requests of up to 1200 tokens, windows of 333 and 150 tokens on the same rows, sharp scores; decoding passes the
+    windows' edges over prompt tokens and decoded ones; four such requests share pages and slots in the mixed schedule."""
+    require_gpu()
+    folder = folders["long_sharp"]
+    requests = rc.random_requests(211, [1200, 400, 700, 3, 520], 21)
+    steps = {"whole": rc.whole, "bulk_tail": lambda r: rc.bulk_tail(r, 200), "portions": lambda r: rc.portions(r, (300, 2, 129, 64, 5, 411, 33)),
+             "mixed": lambda r: rc.mixed(r, seed=3)}[mode](requests)
+    rc.run_replay_inprocess(folder, dtype, str(tmp_path), steps, rc.max_live_tokens(steps), ["--poison-cache"])
+    tol = TOL[dtype] if dtype == "float32" else dict(atol=0.25, rtol=5e-2)
+    rc.compare(rc.collect(str(tmp_path), steps, 211), sc.plain_logits(folder, requests), what="long/%s/%s" % (mode, dtype), **tol)
 
 
 def test_long_decoding_passes_many_windows(folders, tmp_path):
