@@ -5,6 +5,7 @@
 #include <stdint.h>
 #include <stdio.h>
 #include <stdarg.h>
+#include <math.h>
 
 #define SPY_F32 0
 #define SPY_BF16 1
@@ -78,6 +79,12 @@ __device__ __forceinline__ float block_max(float v, float* red) {
     float t = red[0];
     for (int i = 1; i < nw; ++i) t = fmaxf(t, red[i]);
     return t;
+}
+
+// xIELU with the numbers ap = softplus(p), aq = 1/2 + softplus(q):  z > 0: ap z^2 + z/2;  z <= 0: aq (e^z - 1 - z) + z/2
+__device__ __forceinline__ float softplus_f(float x) { return fmaxf(x, 0.f) + log1pf(expf(-fabsf(x))); }
+__device__ __forceinline__ float xielu_f(float z, float ap, float aq) {
+    return z > 0.f ? fmaf(ap * z, z, 0.5f * z) : fmaf(aq, expm1f(z) - z, 0.5f * z);
 }
 
 // Dispatch on a dtype code: binds `T` in `body`.

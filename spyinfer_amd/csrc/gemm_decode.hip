@@ -167,6 +167,10 @@ __global__ __launch_bounds__(GD_WAVES * 64) void gemm_decode_kernel(
         return;
     }
     if (m >= M) return;
+    // the stored product with an activation: w_next, which only the residual epilogue reads otherwise, then points at the
+    // two learned numbers (p, q) of an xIELU that is applied to the result before it is stored
+    const bool act = EPI == EPI_STORE && w_next != nullptr;
+    const float act_p = act ? softplus_f(bf16_to_f32(w_next[0])) : 0.f, act_q = act ? 0.5f + softplus_f(bf16_to_f32(w_next[1])) : 0.f;
     if constexpr (H3) {
         // tile0: all columns (lower) or those of its upper half; the next tile: its lower half, or all
 #pragma unroll
@@ -175,7 +179,7 @@ __global__ __launch_bounds__(GD_WAVES * 64) void gemm_decode_kernel(
             if (!mine) continue;
             TC* out = C + (size_t)m * N + n + 16 * nt;
 #pragma unroll
-            for (int i = 0; i < 4; ++i) out[i] = from_f32<TC>(acc[nt][i]);
+            for (int i = 0; i < 4; ++i) out[i] = from_f32<TC>(act ? xielu_f(acc[nt][i], act_p, act_q) : acc[nt][i]);
         }
         return;
     }
@@ -184,6 +188,7 @@ __global__ __launch_bounds__(GD_WAVES * 64) void gemm_decode_kernel(
     for (int i = 0; i < 4; ++i) {
         float v = acc[0][i];
         if (EPI == EPI_GATED) { const float up = acc[NT - 1][i]; v = (v / (1.0f + expf(-v))) * up; }
+        if (act) v = xielu_f(v, act_p, act_q);
         out[i] = from_f32<TC>(v);
     }
 }
@@ -358,11 +363,15 @@ __global__ __launch_bounds__(GD_WAVES * 64) void gemm_decode_rows_kernel(
                 continue;
             }
             if (m >= M) continue;
+            // (the stored product with an activation: see gemm_decode_kernel)
+            const bool act = EPI == EPI_STORE && w_next != nullptr;
+            const float act_p = act ? softplus_f(bf16_to_f32(w_next[0])) : 0.f, act_q = act ? 0.5f + softplus_f(bf16_to_f32(w_next[1])) : 0.f;
             TC* out = C + (OT ? operand_order(m, n, MT) : (size_t)m * N + n);
 #pragma unroll
             for (int i = 0; i < 4; ++i) {
                 float v = acc[ct][mt][i];
                 if (EPI == EPI_GATED) { const float up = acc[CT + ct][mt][i]; v = (v / (1.0f + expf(-v))) * up; }
+                if (act) v = xielu_f(v, act_p, act_q);
                 out[i] = from_f32<TC>(v);
             }
         }
@@ -469,7 +478,7 @@ extern "C" int64_t spy_gemm_decode_workspace() { return gd_splitk_workspace_byte
 // x: bfloat16 [M, K], M <= 128; MP = 16 times the row tiles the kernel is built with (M rounded up to 16 up to 64 rows, 96
 // or 128 beyond).  scaled != 0: x = bf16(h * w_norm) and ss_in
 // [n_parts, MP] holds the parts of sum(h^2); the result is multiplied by rsqrt(sum / K + eps).
-// epi 0: C [M, N] (c_dtype);  epi 1: W = [gate | up], C [M, N] = silu(gate) * up;  epi 2: resid [M, N] += result,
+// epi 0: C [M, N] (c_dtype), with w_next = two bfloat16 numbers (p, q): xIELU of the result;  epi 1: W = [gate | up], C [M, N] = silu(gate) * up;  epi 2: resid [M, N] += result,
 // xw_out [M, N] = bf16(resid * w_next), ss_out [N / 16, MP] = every block's part of the rows' sums of squares.
 // x_tiled / out_tiled: X / the bfloat16 output for the next product (xw_out of epi 2, C of epi 1) are in operand order.
 extern "C" int spy_gemm_decode(const void* X, int scaled, const float* ss_in, int n_parts, float eps, const void* Wt, int epi,
@@ -490,7 +499,9 @@ extern "C" int spy_gemm_decode(const void* X, int scaled, const float* ss_in, in
     GdArgs a = {(const bf16_t*)X, (const bf16_t*)Wt, C, resid, (bf16_t*)xw_out, (const bf16_t*)w_next, ss_out, ss_in, n_parts, eps, M, N, K,
                 x_tiled != 0, out_tiled != 0, st, ws, (long long)ws_bytes};
     const bool f32 = c_dtype == SPY_F32;
-    if (gd_splitk_try(a, epi, scaled != 0, f32) || gd_wide_try(a, epi, scaled != 0, f32)) {
+    // (a stored product with an activation is built in this file's kernels only)
+    const bool store_act = epi == EPI_STORE && w_next != nullptr;
+    if (!store_act && (gd_splitk_try(a, epi, scaled != 0, f32) || gd_wide_try(a, epi, scaled != 0, f32))) {
         SPY_CHECK_LAUNCH("spy_gemm_decode");
         return 0;
     }

@@ -205,11 +205,7 @@ extern "C" int spy_depth_mix(float* out, void* copy, int copy_dtype, const float
 
 // ---------------------------------------------------------------------------------------------
 // xIELU with the two learned numbers pq = (p, q):  z > 0: softplus(p) z^2 + z/2;  z <= 0: (1/2 + softplus(q)) (e^z - 1 - z) + z/2
-__device__ __forceinline__ float softplus_f(float x) { return fmaxf(x, 0.f) + log1pf(expf(-fabsf(x))); }
-
-__device__ __forceinline__ float xielu_f(float z, float ap, float aq) {
-    return z > 0.f ? fmaf(ap * z, z, 0.5f * z) : fmaf(aq, expm1f(z) - z, 0.5f * z);
-}
+// (softplus_f and xielu_f: common.h, shared with the decode product's store epilogue)
 
 template <typename TA, typename TW>
 __global__ void xielu_kernel(TA* __restrict__ out, const TA* __restrict__ in, const TW* __restrict__ pq, size_t count) {

@@ -504,12 +504,17 @@ def _operand_order_ok(width: int) -> bool:
     return OPERAND_ORDER and width % 32 == 0
 
 
-def decode_linear(x, tiled: torch.Tensor, out_dtype: torch.dtype = torch.bfloat16, out: Optional[torch.Tensor] = None) -> torch.Tensor:
+def decode_linear(x, tiled: torch.Tensor, out_dtype: torch.dtype = torch.bfloat16, out: Optional[torch.Tensor] = None,
+                  xielu_pq: Optional[torch.Tensor] = None) -> torch.Tensor:
     """y = x . w^T for few rows; ``x`` bfloat16 [M, K], OperandRows or a ScaledInput, ``tiled`` from tile_weight; the
-    result goes into ``out`` if one is brought."""
+    result goes into ``out`` if one is brought.  ``xielu_pq``: two bfloat16 numbers (p, q) on the device; the store
+    epilogue then applies the xIELU to the result (up to DECODE_ROWS_PLAIN rows)."""
     N = tiled.shape[0]
     out = _result(out, _rows_of(x), N, out_dtype, tiled.device)
-    _gemm_decode(x, tiled, 0, N, out, None, None, None, None)
+    if xielu_pq is not None:
+        _check(xielu_pq.dtype == torch.bfloat16 and xielu_pq.numel() == 2 and _rows_of(x) <= DECODE_ROWS_PLAIN,
+               "decode_linear: the activation's two numbers must be bfloat16, and the rows at most %d", DECODE_ROWS_PLAIN)
+    _gemm_decode(x, tiled, 0, N, out, None, None, xielu_pq, None)
     return out
 
 
@@ -958,6 +963,9 @@ def xielu(x: torch.Tensor, pq: torch.Tensor) -> torch.Tensor:
 
 def linear_xielu(x: torch.Tensor, w: torch.Tensor, pq: torch.Tensor, tiled: Optional[torch.Tensor] = None) -> torch.Tensor:
     """xielu(x . w^T)."""
+    if (tiled is not None and x.dtype == torch.bfloat16 and pq.dtype == torch.bfloat16 and x.dim() == 2 and 0 < x.shape[0] <= DECODE_ROWS_PLAIN
+            and x.is_contiguous()):
+        return decode_linear(x, tiled, torch.bfloat16, None, pq)           # the activation in the product's store epilogue
     return xielu(linear_few(x, w, tiled), pq)
 
 

@@ -236,6 +236,24 @@ def test_head_products(T, H, N, K, out_dtype):
     assert float(out[:, :, N:].abs().max()) == 0.0
 
 
+@pytest.mark.parametrize("M", [1, 8, 16, 17, 40, 64])
+@pytest.mark.parametrize("N,K", [(256, 256), (3072, 1024), (6144, 512)])
+def test_decode_product_with_the_activation_in_its_epilogue(M, N, K):
+    from spyinfer_amd.kernels import ops
+    dev = require_gpu()
+    g = torch.Generator().manual_seed(8)
+    x = torch.randn((M, K), generator=g).to(torch.bfloat16)
+    w = (torch.randn((N, K), generator=g) / K ** 0.5).to(torch.bfloat16)
+    pq = torch.tensor([0.4, -0.7]).to(torch.bfloat16)
+    tiled = ops.tile_weight(w.to(dev))
+    assert tiled is not None
+    got = ops.linear_xielu(x.to(dev), w.to(dev), pq.to(dev), tiled)
+    ref = plain.xielu(x.double() @ w.double().T, float(pq[0]), float(pq[1]))
+    close(got, ref, torch.bfloat16, what="up product with xIELU, %d rows" % M)
+    # and the same through the separate kernel
+    close(ops.xielu(ops.linear_few(x.to(dev), w.to(dev), tiled), pq.to(dev)), ref, torch.bfloat16, what="product, then xIELU")
+
+
 # ---- whole models under every schedule ------------------------------------------------------------
 MODELS = {"a": (sc.SEF_A, 3, None), "b": (sc.SEF_B, 4, None), "c": (sc.SEF_C, 6, None), "a_sharp": (sc.SEF_A, 5, sc.sharpen()),
           "c_sink": (sc.SEF_C, 9, sc.heavy_sinks()), "long_sharp": (sc.SEF_LONG, 10, sc.sharpen(4.0)),
