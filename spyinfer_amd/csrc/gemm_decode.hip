@@ -52,6 +52,12 @@ __global__ __launch_bounds__(GD_WAVES * 64) void gemm_decode_kernel(
     const bool lower = (blockIdx.x & 1) == 0;                                   // H3: tile0 whole and half of the next, or the reverse
     const int n_base = tile0 * 16;
     const bool x_ok = r < M;                       // lanes whose row of X does not exist load nothing
+    // The stored product with an activation: w_next, which only the residual epilogue reads otherwise, then points at the
+    // two learned numbers (p, q) of an xIELU that is applied to the result before it is stored.  They are asked for now,
+    // with the other loads that the epilogue needs.
+    const bool act = EPI == EPI_STORE && w_next != nullptr;
+    uint32_t act_raw = 0;
+    if (act) act_raw = *reinterpret_cast<const uint32_t*>(w_next);
 
     // Loads whose values are needed only after the product are issued now, so that they are on their way while
     // the matrix streams: every thread's share of the parts of sum(h^2) of row r (the first 256 parts; more are
@@ -167,10 +173,7 @@ __global__ __launch_bounds__(GD_WAVES * 64) void gemm_decode_kernel(
         return;
     }
     if (m >= M) return;
-    // the stored product with an activation: w_next, which only the residual epilogue reads otherwise, then points at the
-    // two learned numbers (p, q) of an xIELU that is applied to the result before it is stored
-    const bool act = EPI == EPI_STORE && w_next != nullptr;
-    const float act_p = act ? softplus_f(bf16_to_f32(w_next[0])) : 0.f, act_q = act ? 0.5f + softplus_f(bf16_to_f32(w_next[1])) : 0.f;
+    const float act_p = act ? softplus_f(__uint_as_float(act_raw << 16)) : 0.f, act_q = act ? 0.5f + softplus_f(__uint_as_float(act_raw & 0xffff0000u)) : 0.f;
     if constexpr (H3) {
         // tile0: all columns (lower) or those of its upper half; the next tile: its lower half, or all
 #pragma unroll
@@ -217,6 +220,9 @@ __global__ __launch_bounds__(GD_WAVES * 64) void gemm_decode_rows_kernel(
     // the wave that will run it (row tile mt belongs to wave mt).
     float ss_part[MT];
     if (SCALED) gd_ss_share<MT, GD_WAVES * 4>(ss_in, n_parts, wave * 4 + g, r, ss_part);
+    const bool act = EPI == EPI_STORE && w_next != nullptr;          // the stored product with an activation: see gemm_decode_kernel
+    uint32_t act_raw = 0;
+    if (act) act_raw = *reinterpret_cast<const uint32_t*>(w_next);
     f32x4_t h_old = {0.f, 0.f, 0.f, 0.f};
     uint2 wn = {0u, 0u};
     if (EPI == EPI_RESID && wave < MT && 16 * wave + r < M) {
@@ -363,9 +369,7 @@ __global__ __launch_bounds__(GD_WAVES * 64) void gemm_decode_rows_kernel(
                 continue;
             }
             if (m >= M) continue;
-            // (the stored product with an activation: see gemm_decode_kernel)
-            const bool act = EPI == EPI_STORE && w_next != nullptr;
-            const float act_p = act ? softplus_f(bf16_to_f32(w_next[0])) : 0.f, act_q = act ? 0.5f + softplus_f(bf16_to_f32(w_next[1])) : 0.f;
+            const float act_p = act ? softplus_f(__uint_as_float(act_raw << 16)) : 0.f, act_q = act ? 0.5f + softplus_f(__uint_as_float(act_raw & 0xffff0000u)) : 0.f;
             TC* out = C + (OT ? operand_order(m, n, MT) : (size_t)m * N + n);
 #pragma unroll
             for (int i = 0; i < 4; ++i) {
@@ -492,6 +496,7 @@ extern "C" int spy_gemm_decode(const void* X, int scaled, const float* ss_in, in
     SPY_REQUIRE(epi != EPI_RESID || (resid && ss_out && xw_out && w_next && ((uintptr_t)resid % 16) == 0 &&
                                      ((uintptr_t)xw_out % 8) == 0 && ((uintptr_t)w_next % 8) == 0),
                 "spy_gemm_decode: the residual epilogue needs the stream, the next norm's weight and its outputs");
+    SPY_REQUIRE(epi != EPI_STORE || !w_next || ((uintptr_t)w_next % 4) == 0, "spy_gemm_decode: the activation's two numbers are not aligned");
     SPY_REQUIRE(epi == EPI_RESID || (C && ((uintptr_t)C % 16) == 0), "spy_gemm_decode: no output");
     SPY_REQUIRE((long long)N * 256 + 8192 < (1ll << 32), "spy_gemm_decode: N = %d is too large for 32-bit offsets inside a chunk", N);
     SPY_REQUIRE(!out_tiled || (N % 32 == 0 && (epi == EPI_RESID || (epi == EPI_GATED && c_dtype == SPY_BF16))),
