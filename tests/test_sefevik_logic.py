@@ -105,7 +105,8 @@ def test_greedy_generation_through_the_entry_point(folders, emu_ops):
     plain = PlainSefevik.from_folder(folder)
     prompts = list(rc.random_requests(97, [5, 17, 2, 30, 9], 9).values())
     want = [plain.greedy(p, 10) for p in prompts]
-    for opts in (dict(), dict(max_num_batched_tokens=12, prefill_chunk=7, max_num_seqs=2)):
+    # (the last: the pool sized from the device's free memory, with the slots' state and the windows' groups counted)
+    for opts in (dict(), dict(max_num_batched_tokens=12, prefill_chunk=7, max_num_seqs=2), dict(num_kvcache_blocks=None)):
         kw = dict(dtype="float32", max_model_len=64, num_kvcache_blocks=24, max_num_seqs=4, kvcache_block_size=8, device="cpu")
         kw.update(opts)
         eng = LLMEngine(folder, **kw)
