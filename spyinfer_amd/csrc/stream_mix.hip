@@ -132,7 +132,23 @@ __global__ void norm_residual_kernel(float* out, TA* __restrict__ copy, const fl
     }
     // Few rows: gridDim.y blocks share a row.  Each forms the whole row's sum of squares (the row is a few kilobytes, from
     // L2) and writes its slice of the outputs, so that a step of a handful of tokens still has blocks for many units.
-    for (int i = threadIdx.x; i < H; i += blockDim.x) { const float v = to_f32<TY>(yr[i]); ss += v * v; }
+    if (sizeof(TY) == 2 && H % 8 == 0 && ((uintptr_t)yr % 16) == 0) {
+        // bfloat16 rows in 16-byte pieces, all of a thread's pieces asked for before the first is squared
+        typedef __attribute__((__vector_size__(4 * sizeof(uint32_t)))) uint32_t u32x4_t;
+        const u32x4_t* y8 = reinterpret_cast<const u32x4_t*>(yr);
+#pragma unroll 4
+        for (int i = threadIdx.x; i < H / 8; i += blockDim.x) {
+            const u32x4_t v = y8[i];
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                const float a = __uint_as_float(v[e] << 16), b = __uint_as_float(v[e] & 0xffff0000u);
+                ss = fmaf(a, a, fmaf(b, b, ss));
+            }
+        }
+    } else {
+#pragma unroll 8
+        for (int i = threadIdx.x; i < H; i += blockDim.x) { const float v = to_f32<TY>(yr[i]); ss += v * v; }
+    }
     ss = block_sum(ss, red);
     const float scale = 1.0f / sqrtf(ss / (float)H + eps);
     const int lo = (int)((long long)H * blockIdx.y / gridDim.y), hi = (int)((long long)H * (blockIdx.y + 1) / gridDim.y);
