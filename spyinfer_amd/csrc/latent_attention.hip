@@ -14,15 +14,24 @@
 // ---------------------------------------------------------------------------------------------
 // Rotation: pair (i, i + dims/2), i < dims/2, of the rotated part; angle = position * freq[i] in float32, cos and sin
 // times `mag`.  Values beyond `dims` pass unchanged.
+#define LP_MAX_PAIRS 512
 template <typename TA, typename TW, typename TQ>
 __global__ void latent_prepare_kernel(TQ* __restrict__ qa, const TA* __restrict__ q, int ldq, const TA* __restrict__ dkv, int ldd,
                                       TA* __restrict__ cache, const int* __restrict__ slot_mapping, long long cache_rows,
                                       const TW* __restrict__ w_norm, float eps, const float* __restrict__ freq, float mag,
                                       int dims, const int* __restrict__ positions, int H, int DN, int DR, int R) {
     __shared__ float red[16];
+    __shared__ float cs[LP_MAX_PAIRS], sn[LP_MAX_PAIRS];
     const int t = blockIdx.x;
     const float p = (float)positions[t];
     const int half = dims / 2;
+    // the token's cos and sin of every rotated pair, once for the block (all heads and the shared key part use them)
+    for (int j = threadIdx.x; j < half; j += blockDim.x) {
+        const float ang = p * freq[j];
+        cs[j] = cosf(ang) * mag;
+        sn[j] = sinf(ang) * mag;
+    }
+    __syncthreads();
     // the heads' rotated parts -> qa[t, h, R ..]
     for (int idx = threadIdx.x; idx < H * DR; idx += blockDim.x) {
         const int h = idx / DR, i = idx - h * DR;
@@ -30,10 +39,8 @@ __global__ void latent_prepare_kernel(TQ* __restrict__ qa, const TA* __restrict_
         float v = to_f32<TA>(src[i]);
         if (i < dims) {
             const int j = i < half ? i : i - half;
-            const float ang = p * freq[j];
-            const float c = cosf(ang) * mag, s = sinf(ang) * mag;
             const float a = to_f32<TA>(src[j]), b = to_f32<TA>(src[j + half]);
-            v = i < half ? a * c - b * s : b * c + a * s;
+            v = i < half ? a * cs[j] - b * sn[j] : b * cs[j] + a * sn[j];
         }
         qa[((size_t)t * H + h) * (R + DR) + R + i] = from_f32<TQ>(v);
     }
@@ -51,10 +58,8 @@ __global__ void latent_prepare_kernel(TQ* __restrict__ qa, const TA* __restrict_
         float v = to_f32<TA>(d[R + i]);
         if (i < dims) {
             const int j = i < half ? i : i - half;
-            const float ang = p * freq[j];
-            const float c = cosf(ang) * mag, s = sinf(ang) * mag;
             const float a = to_f32<TA>(d[R + j]), b = to_f32<TA>(d[R + j + half]);
-            v = i < half ? a * c - b * s : b * c + a * s;
+            v = i < half ? a * cs[j] - b * sn[j] : b * cs[j] + a * sn[j];
         }
         row[R + i] = from_f32<TA>(v);
     }
@@ -65,7 +70,8 @@ extern "C" int spy_latent_prepare(void* qa, int qa_dtype, const void* q, int ldq
                                   const float* freq, float mag, int dims, const int* positions, int T, int H, int DN, int DR, int R,
                                   hipStream_t st) {
     SPY_REQUIRE(T > 0 && H > 0 && DN >= 0 && DR >= 0 && R > 0, "spy_latent_prepare: empty operand");
-    SPY_REQUIRE(dims >= 0 && dims <= DR && dims % 2 == 0 && (dims == 0 || freq), "spy_latent_prepare: %d rotated dims of %d", dims, DR);
+    SPY_REQUIRE(dims >= 0 && dims <= DR && dims % 2 == 0 && (dims == 0 || freq) && dims / 2 <= LP_MAX_PAIRS,
+                "spy_latent_prepare: %d rotated dims of %d (an even number up to %d)", dims, DR, 2 * LP_MAX_PAIRS);
     SPY_REQUIRE(!dkv || (cache && slot_mapping && w_norm), "spy_latent_prepare: storing needs the cache, the tokens' slots and the norm weight");
     SPY_DISPATCH(dtype, TA, SPY_DISPATCH(w_dtype, TW, SPY_DISPATCH(qa_dtype, TQ, (latent_prepare_kernel<TA, TW, TQ><<<T, 256, 0, st>>>(
         (TQ*)qa, (const TA*)q, ldq, (const TA*)dkv, ldd, (TA*)cache, slot_mapping, cache_rows, (const TW*)w_norm, eps, freq, mag, dims,
@@ -447,7 +453,8 @@ __global__ __launch_bounds__(256) void latent_attention_merge_kernel(bf16_t* __r
     __syncthreads();
     for (int j = threadIdx.x; j < R; j += blockDim.x) {
         float o = 0.f;
-        for (int i = 0; i < splits; ++i) o = fmaf(base[(size_t)i * (R + 2) + j], wgt[i], o);
+#pragma unroll 8
+        for (int i = 0; i < splits; ++i) o = fmaf(base[(size_t)i * (R + 2) + j], wgt[i], o);      // (unrolled: the parts' loads go out together)
         out[row * R + j] = f32_to_bf16(o * inv_l);
     }
 }

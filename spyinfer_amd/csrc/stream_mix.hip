@@ -53,6 +53,35 @@ __global__ void pair_embedding_kernel(float* __restrict__ out, TA* __restrict__ 
         prow = pair + (size_t)pair_row * H;
         if (threadIdx.x == 0 && t == first && slot >= 0 && slot < num_slots) last_token[slot] = ids[cu_q[e + 1] - 1];
     }
+    if (sizeof(TW) == 2 && H % 8 == 0 && ((uintptr_t)row % 16) == 0 && (!prow || ((uintptr_t)prow % 16) == 0) && ((uintptr_t)o % 16) == 0 &&
+        (!c || ((uintptr_t)c % 16) == 0)) {
+        // bfloat16 tables: 8 values a thread and step, 16-byte loads of both rows asked for together
+        typedef __attribute__((__vector_size__(4 * sizeof(uint32_t)))) uint32_t u32x4_t;
+        typedef __attribute__((__vector_size__(4 * sizeof(float)))) float f4_t;
+#pragma unroll 2
+        for (int i = threadIdx.x * 8; i < H; i += blockDim.x * 8) {
+            const u32x4_t a = *reinterpret_cast<const u32x4_t*>(row + i);
+            u32x4_t b = {0u, 0u, 0u, 0u};
+            if (prow) b = *reinterpret_cast<const u32x4_t*>(prow + i);
+            float v[8];
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                v[2 * e] = __uint_as_float(a[e] << 16) + __uint_as_float(b[e] << 16);
+                v[2 * e + 1] = __uint_as_float(a[e] & 0xffff0000u) + __uint_as_float(b[e] & 0xffff0000u);
+            }
+            *reinterpret_cast<f4_t*>(o + i) = f4_t{v[0], v[1], v[2], v[3]};
+            *reinterpret_cast<f4_t*>(o + i + 4) = f4_t{v[4], v[5], v[6], v[7]};
+            if (c) {
+                if (sizeof(TA) == 2) {
+                    *reinterpret_cast<u32x4_t*>(c + i) = u32x4_t{pack_bf16x2(v[0], v[1]), pack_bf16x2(v[2], v[3]), pack_bf16x2(v[4], v[5]), pack_bf16x2(v[6], v[7])};
+                } else {
+#pragma unroll
+                    for (int e = 0; e < 8; ++e) c[i + e] = from_f32<TA>(v[e]);
+                }
+            }
+        }
+        return;
+    }
     for (int i = threadIdx.x; i < H; i += blockDim.x) {
         float v = to_f32<TW>(row[i]);
         if (prow) v += to_f32<TW>(prow[i]);
