@@ -112,3 +112,9 @@ def test_greedy_generation_through_the_entry_point(folders, emu_ops):
         eng = LLMEngine(folder, **kw)
         assert eng.generate(prompts, SamplingParams(max_new_tokens=10, ignore_eos=True)) == want
         eng.runner.manager.check()
+    # a pool too small for all requests at once: the request admitted last is preempted, gives its slot and pages back
+    # and later runs again from its first token, with the recurrences' state and the previous token starting anew
+    eng = LLMEngine(folder, dtype="float32", max_model_len=64, num_kvcache_blocks=9, max_num_seqs=4, kvcache_block_size=8, device="cpu")
+    assert eng.generate(prompts, SamplingParams(max_new_tokens=10, ignore_eos=True)) == want
+    assert eng.scheduler.num_preemptions > 0
+    eng.runner.manager.check()
