@@ -4,10 +4,13 @@
 // head's output is Wuv_h (sum_j p_j c_j).  So the kernels here see one "key" row of R + DR values and one "value" row of
 // R values (its first part) per token and H query rows per token against them.
 //
-//   spy_latent_prepare    c = rmsnorm(dkv[:R]) * w and kr = rotate(dkv[R:]) into the pages; the heads' rotated query parts
-//                         into the absorbed query rows
-//   spy_gemm_strided      batched product with element strides (the per-head products with Wuk and Wuv), float32 sums
-//   spy_latent_attention  plain kernel, float32: one block per (token, head); softmax with a sink in the denominator
+//   spy_latent_prepare         c = rmsnorm(dkv[:R]) * w and kr = rotate(dkv[R:]) into the pages; the heads' rotated query
+//                              parts into the absorbed query rows
+//   spy_head_products          the per-head products with Wuk and Wuv on MFMA, few rows (many rows: the library's batched product)
+//   spy_latent_attention_mfma  bfloat16: 64 or 128 query rows a block against key chunks staged once in LDS; keys in parts for
+//                              steps of single tokens, merged by a second kernel
+//   spy_latent_attention       plain kernel, float32: one block per (token, head); the same window and sink
+//   spy_gemm_strided           batched product with element strides, float32 sums (the float32 path's per-head products)
 #include "common.h"
 #include <math.h>
 

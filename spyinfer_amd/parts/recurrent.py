@@ -8,6 +8,7 @@ starts at zero, is float32 and lives in the request's slot; everything behind th
 from __future__ import annotations
 
 import numpy as np
+import torch
 
 from ..cache.spec import FixedState
 from ..kernels import ops
@@ -55,7 +56,6 @@ class MinGRU(Mixer):
         if len({m.dtype for m in mats}) > 1:
             mats = [m.float() for m in mats]
         # one product for the three projections: rows [z | x | g]
-        import torch
         self.w_zxg, self.w_zxg_tiled = ops.weight_forms(torch.cat(mats, dim=0).contiguous())
         del mats
         self.w_o, self.w_o_tiled = ops.weight_forms(weights.pop(o))
