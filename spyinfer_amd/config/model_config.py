@@ -286,3 +286,120 @@ class SefevikConfig(ModelConfig):
                 if (other["kv_rank"], other["rot_dim"], other["rot"]) != (m["kv_rank"], m["rot_dim"], m["rot"]):
                     raise ConfigError("config.json layers[%d].mixer: kv_rank, rot_dim and rot must equal those of layer %d, "
                                       "whose cache it reads" % (i, src))
+
+
+@dataclasses.dataclass
+class SodedraConfig(ModelConfig):
+    """Sodedra: layers whose two sublayers read one norm of the stream (weights stored around zero) and are added
+    together; token mixers 'mlstm' (a matrix memory with exponential gates), 'attention' (grouped queries, projection
+    biases, heads rotated in part with frequencies rescaled by wavelength, a sliding window, a sigmoid gate on the
+    result) and 'channel_delta' (a gated delta rule with short convolutions and a decay per key channel); feed-forwards
+    'dense' (gated) or 'moe' (a mixture of gated experts chosen among the best groups); a scaled embedding whose table is
+    also the output head.  The configuration is nested; ``layers`` lists every layer's type and sizes, and nothing is
+    assumed equal between layers."""
+
+    architecture: str = ""
+    vocab: int = -1
+    width: int = -1
+    norm_eps: float = 0.0
+    embedding_scale: float = 1.0
+    #: one dict per layer: type, mixer (sizes and constants of that mixer), mlp (None, {kind: dense, ff} or
+    #: {kind: moe, ff, experts, top, groups, keep, scale})
+    layers: List[Dict[str, Any]] = dataclasses.field(default_factory=list)
+
+    MIXERS: ClassVar[tuple] = ("mlstm", "attention", "channel_delta")
+
+    @classmethod
+    def from_dict(cls, raw: Dict[str, Any]) -> "SodedraConfig":
+        cfg = cls(architecture=str(raw.get("architecture") or (raw.get("architectures") or [""])[0]),
+                  vocab=_need(raw, "vocab", int), width=_need(raw, "width", int), norm_eps=float(_need(raw, "norm.eps", (int, float))))
+        if (raw.get("embedding") or {}).get("scale") is not None:
+            cfg.embedding_scale = float(_need(raw, "embedding.scale", (int, float)))
+        cfg.layers = [cls._layer(i, l) for i, l in enumerate(_need(raw, "layers", list))]
+        cfg._raw = dict(raw)
+        cfg.validate()
+        return cfg
+
+    @classmethod
+    def _layer(cls, i: int, raw: Dict[str, Any]) -> Dict[str, Any]:
+        where = "config.json layers[%d]" % i
+        if not isinstance(raw, dict):
+            raise ConfigError("%s is no object" % where)
+        kind = _need(raw, "type", str, where)
+        if kind not in cls.MIXERS:
+            raise ConfigError("%s: mixer type %r is not known (%s)" % (where, kind, ", ".join(cls.MIXERS)))
+        m = _need(raw, "mixer", dict, where)
+        at = where + ".mixer"
+        if kind == "mlstm":
+            mix = {k: _need(m, k, int, at) for k in ("heads", "dim", "vdim")}
+            mix["gate_cap"] = float(_need(m, "gate_cap", (int, float), at))
+        elif kind == "attention":
+            mix = {k: _need(m, k, int, at) for k in ("heads", "kv_heads", "dim", "vdim")}
+            mix["scale"] = float(_need(m, "scale", (int, float), at))
+            mix["window"] = _need(m, "mask.size", int, at) if m.get("mask") else None
+            rot = m.get("rot")
+            mix["rot"] = None
+            if rot:
+                mix["rot"] = {"base": float(_need(rot, "base", (int, float), at + ".rot")), "dims": _need(rot, "dims", int, at + ".rot"),
+                              "scaling": None}
+                sc = rot.get("scaling")
+                if sc:
+                    mix["rot"]["scaling"] = {k: float(_need(sc, k, (int, float), at + ".rot.scaling")) for k in ("factor", "low", "high", "original")}
+        else:
+            mix = {k: _need(m, k, int, at) for k in ("heads", "kv_heads", "dim", "vdim", "conv")}
+            # inner sizes of the low-rank projections: no key of the design; the stored tensors decide unless these are given
+            for k in ("decay_rank", "gate_rank"):
+                mix[k] = _need(m, k, int, at) if m.get(k) is not None else None
+        out = {"type": kind, "mixer": mix, "mlp": None}
+        mlp = raw.get("mlp")
+        if mlp is not None:
+            at = where + ".mlp"
+            fk = _need(mlp, "kind", str, at)
+            if fk == "dense":
+                out["mlp"] = {"kind": fk, "ff": _need(mlp, "ff", int, at)}
+            elif fk == "moe":
+                groups = (mlp.get("router") or {}).get("groups")
+                out["mlp"] = {"kind": fk, "ff": _need(mlp, "expert.ff", int, at), "experts": _need(mlp, "router.experts", int, at),
+                              "top": _need(mlp, "router.top", int, at),
+                              "groups": _need(groups, "count", int, at + ".router.groups") if groups else 1,
+                              "keep": _need(groups, "keep", int, at + ".router.groups") if groups else 1,
+                              "scale": float(_need(mlp, "router.scale", (int, float), at)) if (mlp.get("router") or {}).get("scale") is not None else 1.0}
+            else:
+                raise ConfigError("%s: kind %r is not known (dense, moe)" % (at, fk))
+        return out
+
+    def to_dict(self) -> Dict[str, Any]:
+        return dict(getattr(self, "_raw", {}))
+
+    def validate(self) -> None:
+        if self.vocab <= 0 or self.width <= 0:
+            raise ConfigError("config.json: vocab and width must be positive")
+        if not (self.norm_eps > 0.0):
+            raise ConfigError("config.json: norm.eps must be positive")
+        if not self.layers:
+            raise ConfigError("config.json: no layers")
+        for i, layer in enumerate(self.layers):
+            m, where = layer["mixer"], "config.json layers[%d]" % i
+            if any(isinstance(v, int) and not isinstance(v, bool) and v <= 0 for v in m.values()):
+                raise ConfigError("%s.mixer: sizes must be positive" % where)
+            if "kv_heads" in m and m["heads"] % m["kv_heads"]:
+                raise ConfigError("%s.mixer: heads (%d) is not a multiple of kv_heads (%d)" % (where, m["heads"], m["kv_heads"]))
+            if layer["type"] == "mlstm" and not m["gate_cap"] > 0.0:
+                raise ConfigError("%s.mixer.gate_cap must be positive" % where)
+            if layer["type"] == "channel_delta" and m["conv"] > 8:
+                raise ConfigError("%s.mixer.conv: at most 8 taps" % where)
+            if layer["type"] == "attention" and m["rot"]:
+                rot = m["rot"]
+                if rot["dims"] % 2 or not (0 < rot["dims"] <= m["dim"]) or not rot["base"] > 1.0:
+                    raise ConfigError("%s.mixer.rot: dims must be even and at most dim, base above 1" % where)
+                sc = rot["scaling"]
+                if sc and not (sc["factor"] > 0.0 and sc["original"] > 0.0 and 0.0 < sc["low"] <= sc["high"]):
+                    raise ConfigError("%s.mixer.rot.scaling: factor and original positive, 0 < low <= high" % where)
+            f = layer["mlp"]
+            if f and f["ff"] <= 0:
+                raise ConfigError("%s.mlp: the inner size must be positive" % where)
+            if f and f["kind"] == "moe":
+                E, G = f["experts"], f["groups"]
+                if E <= 0 or G <= 0 or E % G or not 0 < f["keep"] <= G or not 0 < f["top"] <= f["keep"] * (E // G):
+                    raise ConfigError("%s.mlp.router: %d choices among %d of %d groups of %d experts cannot be made"
+                                      % (where, f["top"], f["keep"], G, E))

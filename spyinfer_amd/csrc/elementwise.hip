@@ -4,9 +4,10 @@
 #include "common.h"
 
 // ---------------------------------------------------------------------------------------------
-// out[t, :] = table[ids[t], :]  (float32 out: the start of the residual stream)
+// out[t, :] = table[ids[t], :] * scale  (float32 out: the start of the residual stream)
 template <typename TW>
-__global__ void embedding_kernel(float* __restrict__ out, const TW* __restrict__ table, const int* __restrict__ ids, int H, int V) {
+__global__ void embedding_kernel(float* __restrict__ out, const TW* __restrict__ table, const int* __restrict__ ids, int H, int V,
+                                 float scale) {
     const int t = blockIdx.x;
     const int id = ids[t];
     float* o = out + (size_t)t * H;
@@ -15,12 +16,13 @@ __global__ void embedding_kernel(float* __restrict__ out, const TW* __restrict__
         return;
     }
     const TW* row = table + (size_t)id * H;
-    for (int i = threadIdx.x; i < H; i += blockDim.x) o[i] = to_f32<TW>(row[i]);
+    for (int i = threadIdx.x; i < H; i += blockDim.x) o[i] = to_f32<TW>(row[i]) * scale;
 }
 
-extern "C" int spy_embedding(float* out, const void* table, int table_dtype, const int* ids, int T, int H, int V, hipStream_t st) {
+extern "C" int spy_embedding(float* out, const void* table, int table_dtype, const int* ids, int T, int H, int V, float scale,
+                             hipStream_t st) {
     SPY_REQUIRE(T > 0 && H > 0 && V > 0, "spy_embedding: empty operand");
-    SPY_DISPATCH(table_dtype, TW, embedding_kernel<TW><<<T, 256, 0, st>>>(out, (const TW*)table, ids, H, V));
+    SPY_DISPATCH(table_dtype, TW, embedding_kernel<TW><<<T, 256, 0, st>>>(out, (const TW*)table, ids, H, V, scale));
     SPY_CHECK_LAUNCH("spy_embedding");
     return 0;
 }
@@ -100,7 +102,8 @@ extern "C" int spy_embedding_sumsq(float* out, void* xw, float* ss, const void* 
 }
 
 // ---------------------------------------------------------------------------------------------
-// x = resid[t] (+ delta[t]);  rows == null: resid[t] = x.  out[r] = (x / sqrt(mean(x^2) + eps)) * w
+// x = resid[t] (+ delta[t] (+ delta2[t]));  rows == null: resid[t] = x.  out[r] = (x / sqrt(mean(x^2) + eps)) * w
+// (two addends: the results of two sublayers that read the same norm, summed in float32 before they meet the stream)
 // One block per row.  The row is read once and kept in registers (4 values per thread and pass,
 // up to NORM_PASSES passes); longer rows are read again for the second pass.
 #define NORM_PASSES 8
@@ -125,8 +128,9 @@ template <> struct Vec4<bf16_t> {
 };
 
 template <typename TA, typename TW, bool VEC>
-__global__ void add_rmsnorm_kernel(float* __restrict__ resid, const TA* __restrict__ delta, const TW* __restrict__ w, float eps,
-                                   TA* __restrict__ out, const int* __restrict__ rows, int T, int H) {
+__global__ void add_rmsnorm_kernel(float* __restrict__ resid, const TA* __restrict__ delta, const TA* __restrict__ delta2,
+                                   const TW* __restrict__ w, float eps, TA* __restrict__ out, const int* __restrict__ rows, int T,
+                                   int H) {
     __shared__ float red[16];
     const int r = blockIdx.x;
     int t = r;
@@ -139,6 +143,7 @@ __global__ void add_rmsnorm_kernel(float* __restrict__ resid, const TA* __restri
     }
     float* x = resid + (size_t)t * H;
     const TA* dl = delta ? delta + (size_t)t * H : nullptr;
+    const TA* dl2 = delta2 ? delta2 + (size_t)t * H : nullptr;
     TA* o = out + (size_t)r * H;
     const bool write_back = dl && !rows;
     if (VEC) {
@@ -153,6 +158,12 @@ __global__ void add_rmsnorm_kernel(float* __restrict__ resid, const TA* __restri
                 if (dl) {
                     float d4[4];
                     Vec4<TA>::load(dl + i, d4);
+                    if (dl2) {
+                        float e4[4];
+                        Vec4<TA>::load(dl2 + i, e4);
+#pragma unroll
+                        for (int e = 0; e < 4; ++e) d4[e] += e4[e];
+                    }
 #pragma unroll
                     for (int e = 0; e < 4; ++e) v[p][e] += d4[e];
                 }
@@ -179,7 +190,7 @@ __global__ void add_rmsnorm_kernel(float* __restrict__ resid, const TA* __restri
     float ss = 0.f;
     for (int i = threadIdx.x; i < H; i += blockDim.x) {
         float v = x[i];
-        if (dl) v += to_f32<TA>(dl[i]);
+        if (dl) v += to_f32<TA>(dl[i]) + (dl2 ? to_f32<TA>(dl2[i]) : 0.f);
         if (write_back) x[i] = v;
         ss += v * v;
     }
@@ -187,24 +198,25 @@ __global__ void add_rmsnorm_kernel(float* __restrict__ resid, const TA* __restri
     const float scale = 1.0f / sqrtf(ss / (float)H + eps);
     for (int i = threadIdx.x; i < H; i += blockDim.x) {
         float v = x[i];
-        if (dl && rows) v += to_f32<TA>(dl[i]);
+        if (dl && rows) v += to_f32<TA>(dl[i]) + (dl2 ? to_f32<TA>(dl2[i]) : 0.f);
         o[i] = from_f32<TA>((scale * v) * to_f32<TW>(w[i]));
     }
 }
 
-extern "C" int spy_add_rmsnorm(float* resid, const void* delta, const void* w, int w_dtype, float eps, void* out, int out_dtype,
-                               const int* rows, int n_out, int T, int H, hipStream_t st) {
+extern "C" int spy_add_rmsnorm(float* resid, const void* delta, const void* delta2, const void* w, int w_dtype, float eps, void* out,
+                               int out_dtype, const int* rows, int n_out, int T, int H, hipStream_t st) {
     SPY_REQUIRE(n_out > 0 && T > 0 && H > 0, "spy_add_rmsnorm: empty operand");
+    SPY_REQUIRE(delta || !delta2, "spy_add_rmsnorm: a second addend without a first");
     const int threads = H >= 2048 ? 256 : (H >= 512 ? 128 : 64);
-    const bool aligned = H % 4 == 0 && ((uintptr_t)resid % 16) == 0 && ((uintptr_t)delta % 16) == 0 && ((uintptr_t)w % 16) == 0 &&
+    const bool aligned = H % 4 == 0 && ((uintptr_t)resid % 16) == 0 && ((uintptr_t)delta % 16) == 0 && ((uintptr_t)delta2 % 16) == 0 && ((uintptr_t)w % 16) == 0 &&
                          ((uintptr_t)out % 16) == 0;
     const bool vec = aligned && H <= threads * 4 * NORM_PASSES;
     if (vec) {
         SPY_DISPATCH(out_dtype, TA, SPY_DISPATCH(w_dtype, TW, (add_rmsnorm_kernel<TA, TW, true><<<n_out, threads, 0, st>>>(
-            resid, (const TA*)delta, (const TW*)w, eps, (TA*)out, rows, T, H))));
+            resid, (const TA*)delta, (const TA*)delta2, (const TW*)w, eps, (TA*)out, rows, T, H))));
     } else {
         SPY_DISPATCH(out_dtype, TA, SPY_DISPATCH(w_dtype, TW, (add_rmsnorm_kernel<TA, TW, false><<<n_out, 512, 0, st>>>(
-            resid, (const TA*)delta, (const TW*)w, eps, (TA*)out, rows, T, H))));
+            resid, (const TA*)delta, (const TA*)delta2, (const TW*)w, eps, (TA*)out, rows, T, H))));
     }
     SPY_CHECK_LAUNCH("spy_add_rmsnorm");
     return 0;

@@ -1,0 +1,253 @@
+// Mixture of experts: the router's choice, the (token, choice) pairs sorted by expert, the experts' products over the
+// sorted rows, and the weighted sum of a token's results.  Nothing here needs the host to know how many tokens an
+// expert got: the sizes of all arrays follow the number of tokens alone, and blocks whose tile holds no rows leave.
+//
+//   route:   s = softmax(z) over all experts (float32); choice = s + correction; the experts form `groups` equal runs of
+//            neighbours, a group's score is its largest choice, only experts of the `keep` best groups can be chosen (the
+//            others count as minus infinity); the `top` largest choices are taken; their weights are s (without the
+//            correction) over their sum (+ 1e-20), times `scale`.
+//   align:   rows of the sorted order: expert e's pairs in a run that starts at a multiple of MOE_TM rows, padded with -1.
+//   gemm:    C[row] = A[source of row] . W[expert of the row's tile]^T, float32 products and sums; optionally gated:
+//            W = [gate rows | up rows], C = silu(gate) * up.
+//   combine: out[t] = sum_k weight[t, k] * Y[row of pair (t, k)].
+#include "common.h"
+#include <math.h>
+
+#define MOE_TM 16
+#define MOE_MAX_EXPERTS 1024
+
+// one wave per token
+__global__ __launch_bounds__(64) void moe_route_kernel(int* __restrict__ ids, float* __restrict__ weights, const float* __restrict__ z,
+                                                       const float* __restrict__ correction, int E, int top, int groups, int keep,
+                                                       float scale) {
+    __shared__ float sc[MOE_MAX_EXPERTS], ch[MOE_MAX_EXPERTS], gsc[MOE_MAX_EXPERTS];
+    __shared__ int allowed[MOE_MAX_EXPERTS], sel[MOE_MAX_EXPERTS];
+    const int t = blockIdx.x, lane = threadIdx.x;
+    const float* zr = z + (size_t)t * E;
+    float mx = -INFINITY;
+    for (int e = lane; e < E; e += 64) mx = fmaxf(mx, zr[e]);
+    mx = wave_max(mx);
+    float sum = 0.f;
+    for (int e = lane; e < E; e += 64) {
+        const float p = expf(zr[e] - mx);
+        sc[e] = p;
+        sum += p;
+    }
+    sum = wave_sum(sum);
+    for (int e = lane; e < E; e += 64) {
+        sc[e] = sc[e] / sum;
+        ch[e] = sc[e] + correction[e];
+    }
+    __syncthreads();
+    const int per = E / groups;
+    for (int g = lane; g < groups; g += 64) {
+        float best = -INFINITY;
+        for (int i = 0; i < per; ++i) best = fmaxf(best, ch[g * per + i]);
+        gsc[g] = best;
+        allowed[g] = 0;
+    }
+    __syncthreads();
+    for (int r = 0; r < keep; ++r) {
+        float bv = -INFINITY;
+        int bi = 0x7fffffff;
+        for (int g = lane; g < groups; g += 64)
+            if (!allowed[g] && (gsc[g] > bv || (gsc[g] == bv && g < bi))) { bv = gsc[g]; bi = g; }
+#pragma unroll
+        for (int o = 32; o > 0; o >>= 1) {
+            const float ov = __shfl_xor(bv, o, 64);
+            const int oi = __shfl_xor(bi, o, 64);
+            if (ov > bv || (ov == bv && oi < bi)) { bv = ov; bi = oi; }
+        }
+        if (lane == 0 && bi < groups) allowed[bi] = 1;
+        __syncthreads();
+    }
+    for (int e = lane; e < E; e += 64)
+        if (!allowed[e / per]) ch[e] = -INFINITY;
+    __syncthreads();
+    float wsum = 0.f;
+    for (int r = 0; r < top; ++r) {
+        float bv = -INFINITY;
+        int bi = 0x7fffffff;
+        for (int e = lane; e < E; e += 64)
+            if (ch[e] > bv) { bv = ch[e]; bi = e; }
+#pragma unroll
+        for (int o = 32; o > 0; o >>= 1) {
+            const float ov = __shfl_xor(bv, o, 64);
+            const int oi = __shfl_xor(bi, o, 64);
+            if (ov > bv || (ov == bv && oi < bi)) { bv = ov; bi = oi; }
+        }
+        if (bi >= E) bi = 0;                       // fewer allowed experts than choices: never the case for a checked configuration
+        wsum += sc[bi];
+        __syncthreads();
+        if (lane == 0) { ch[bi] = -INFINITY; sel[r] = bi; }
+        __syncthreads();
+    }
+    const float norm = scale / (wsum + 1e-20f);
+    for (int r = lane; r < top; r += 64) {
+        ids[(size_t)t * top + r] = sel[r];
+        weights[(size_t)t * top + r] = sc[sel[r]] * norm;
+    }
+}
+
+extern "C" int spy_moe_route(int* ids, float* weights, const float* z, const float* correction, int T, int E, int top, int groups,
+                             int keep, float scale, hipStream_t st) {
+    SPY_REQUIRE(T > 0 && E > 0 && E <= MOE_MAX_EXPERTS, "spy_moe_route: %d experts (1..%d)", E, MOE_MAX_EXPERTS);
+    SPY_REQUIRE(groups > 0 && E % groups == 0 && keep > 0 && keep <= groups && top > 0 && top <= keep * (E / groups),
+                "spy_moe_route: %d of %d groups of %d experts cannot give %d choices", keep, groups, E / (groups > 0 ? groups : 1), top);
+    moe_route_kernel<<<T, 64, 0, st>>>(ids, weights, z, correction, E, top, groups, keep, scale);
+    SPY_CHECK_LAUNCH("spy_moe_route");
+    return 0;
+}
+
+// One block.  ids [P] -> sorted_pair [max_tiles MOE_TM] (pair or -1), pair_row [P], tile_expert [max_tiles] (expert or -1).
+__global__ __launch_bounds__(1024) void moe_align_kernel(int* __restrict__ sorted_pair, int* __restrict__ pair_row,
+                                                         int* __restrict__ tile_expert, const int* __restrict__ ids, int P, int E,
+                                                         int max_tiles) {
+    __shared__ int count[MOE_MAX_EXPERTS], first[MOE_MAX_EXPERTS], cursor[MOE_MAX_EXPERTS];
+    __shared__ int total_tiles;
+    const int tid = threadIdx.x;
+    for (int e = tid; e < E; e += blockDim.x) { count[e] = 0; cursor[e] = 0; }
+    __syncthreads();
+    for (int p = tid; p < P; p += blockDim.x) {
+        const int e = ids[p];
+        if (e >= 0 && e < E) atomicAdd(&count[e], 1);
+    }
+    __syncthreads();
+    if (tid == 0) {
+        int tiles = 0;
+        for (int e = 0; e < E; ++e) {
+            first[e] = tiles;
+            tiles += (count[e] + MOE_TM - 1) / MOE_TM;
+        }
+        total_tiles = tiles;
+    }
+    __syncthreads();
+    for (int e = tid; e < E; e += blockDim.x) {
+        const int nt = (count[e] + MOE_TM - 1) / MOE_TM;
+        for (int i = 0; i < nt && first[e] + i < max_tiles; ++i) tile_expert[first[e] + i] = e;
+        for (int r = count[e]; r < nt * MOE_TM; ++r)
+            if (first[e] * MOE_TM + r < max_tiles * MOE_TM) sorted_pair[first[e] * MOE_TM + r] = -1;
+    }
+    for (int i = total_tiles + tid; i < max_tiles; i += blockDim.x) tile_expert[i] = -1;
+    for (int r = total_tiles * MOE_TM + tid; r < max_tiles * MOE_TM; r += blockDim.x) sorted_pair[r] = -1;
+    for (int p = tid; p < P; p += blockDim.x) {
+        const int e = ids[p];
+        if (e < 0 || e >= E) { pair_row[p] = -1; continue; }
+        const int row = first[e] * MOE_TM + atomicAdd(&cursor[e], 1);
+        if (row < max_tiles * MOE_TM) sorted_pair[row] = p;
+        pair_row[p] = row < max_tiles * MOE_TM ? row : -1;
+    }
+}
+
+extern "C" int spy_moe_align(int* sorted_pair, int* pair_row, int* tile_expert, const int* ids, int P, int E, int max_tiles,
+                             hipStream_t st) {
+    SPY_REQUIRE(P > 0 && E > 0 && E <= MOE_MAX_EXPERTS, "spy_moe_align: %d experts (1..%d)", E, MOE_MAX_EXPERTS);
+    SPY_REQUIRE(max_tiles >= P / MOE_TM + (E < P ? E : P), "spy_moe_align: %d tiles are too few for %d pairs of %d experts", max_tiles, P, E);
+    moe_align_kernel<<<1, 1024, 0, st>>>(sorted_pair, pair_row, tile_expert, ids, P, E, max_tiles);
+    SPY_CHECK_LAUNCH("spy_moe_align");
+    return 0;
+}
+
+extern "C" int spy_moe_tile_rows() { return MOE_TM; }
+
+// A tile of MOE_TM sorted rows x 64 columns per block; 256 threads, thread (ty, tx) has row ty and columns 4 tx .. + 3.
+// gather > 0: row r reads A[sorted_pair[r] / gather] (the token of the pair); 0: A[r].
+#define MG_TN 64
+#define MG_K 16
+template <typename TA, typename TW, typename TC, bool GATED>
+__global__ __launch_bounds__(256) void moe_gemm_kernel(TC* __restrict__ C, const TA* __restrict__ A, const TW* __restrict__ W,
+                                                       const int* __restrict__ tile_expert, const int* __restrict__ sorted_pair,
+                                                       int gather, int N, int K, long long w_stride) {
+    __shared__ float As[MG_K][MOE_TM + 1];
+    __shared__ float Ws[GATED ? 2 : 1][MG_K][MG_TN + 4];
+    __shared__ int src[MOE_TM];
+    const int tile = blockIdx.y;
+    const int e = tile_expert[tile];
+    if (e < 0) return;
+    const int n0 = blockIdx.x * MG_TN;
+    const int tx = threadIdx.x & 15, ty = threadIdx.x >> 4;
+    if (threadIdx.x < MOE_TM) {
+        const int p = sorted_pair[tile * MOE_TM + threadIdx.x];
+        src[threadIdx.x] = p < 0 ? -1 : (gather > 0 ? p / gather : tile * MOE_TM + (int)threadIdx.x);
+    }
+    __syncthreads();
+    const TW* We = W + (size_t)e * w_stride;
+    float acc[4] = {}, acc2[4] = {};
+    // staging: A 16 x 16 values, one per thread; W 64 x 16 values, four per thread
+    const int ar = threadIdx.x >> 4, ak = threadIdx.x & 15;
+    const int wr = threadIdx.x >> 2, wk = (threadIdx.x & 3) * 4;
+    for (int k0 = 0; k0 < K; k0 += MG_K) {
+        {
+            const int sr = src[ar], k = k0 + ak;
+            As[ak][ar] = (sr >= 0 && k < K) ? to_f32<TA>(A[(size_t)sr * K + k]) : 0.f;
+        }
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const int k = k0 + wk + i, n = n0 + wr;
+            Ws[0][wk + i][wr] = (n < N && k < K) ? to_f32<TW>(We[(size_t)n * K + k]) : 0.f;
+            if (GATED) Ws[GATED ? 1 : 0][wk + i][wr] = (n < N && k < K) ? to_f32<TW>(We[(size_t)(N + n) * K + k]) : 0.f;
+        }
+        __syncthreads();
+#pragma unroll
+        for (int k = 0; k < MG_K; ++k) {
+            const float a = As[k][ty];
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                acc[i] = fmaf(a, Ws[0][k][tx * 4 + i], acc[i]);
+                if (GATED) acc2[i] = fmaf(a, Ws[GATED ? 1 : 0][k][tx * 4 + i], acc2[i]);
+            }
+        }
+        __syncthreads();
+    }
+    if (src[ty] < 0) return;
+    const size_t row = (size_t)tile * MOE_TM + ty;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        const int n = n0 + tx * 4 + i;
+        if (n >= N) continue;
+        float v = acc[i];
+        if (GATED) {
+            v = acc[i] / (1.0f + expf(-acc[i])) * acc2[i];
+        }
+        C[row * N + n] = from_f32<TC>(v);
+    }
+}
+
+extern "C" int spy_moe_gemm(void* C, int c_dtype, const void* A, int a_dtype, const void* W, int w_dtype, const int* tile_expert,
+                            const int* sorted_pair, int gather, int gated, int max_tiles, int E, int N, int K, hipStream_t st) {
+    SPY_REQUIRE(max_tiles > 0 && max_tiles <= 65535 && E > 0 && N > 0 && K > 0 && gather >= 0, "spy_moe_gemm: bad sizes (%d tiles)", max_tiles);
+    const dim3 grid((N + MG_TN - 1) / MG_TN, max_tiles);
+    const long long ws = (long long)(gated ? 2 : 1) * N * K;
+    if (gated) {
+        SPY_DISPATCH(a_dtype, TA, SPY_DISPATCH(w_dtype, TW, SPY_DISPATCH(c_dtype, TC, (moe_gemm_kernel<TA, TW, TC, true><<<grid, 256, 0, st>>>(
+            (TC*)C, (const TA*)A, (const TW*)W, tile_expert, sorted_pair, gather, N, K, ws)))));
+    } else {
+        SPY_DISPATCH(a_dtype, TA, SPY_DISPATCH(w_dtype, TW, SPY_DISPATCH(c_dtype, TC, (moe_gemm_kernel<TA, TW, TC, false><<<grid, 256, 0, st>>>(
+            (TC*)C, (const TA*)A, (const TW*)W, tile_expert, sorted_pair, gather, N, K, ws)))));
+    }
+    SPY_CHECK_LAUNCH("spy_moe_gemm");
+    return 0;
+}
+
+// out[t, :] = sum_k weights[t, k] * Y[pair_row[t top + k], :], added in ascending k
+template <typename TC>
+__global__ void moe_combine_kernel(TC* __restrict__ out, const float* __restrict__ Y, const float* __restrict__ weights,
+                                   const int* __restrict__ pair_row, int top, int H) {
+    const int t = blockIdx.x;
+    for (int c = threadIdx.x; c < H; c += blockDim.x) {
+        float acc = 0.f;
+        for (int k = 0; k < top; ++k) {
+            const int row = pair_row[(size_t)t * top + k];
+            if (row >= 0) acc = fmaf(weights[(size_t)t * top + k], Y[(size_t)row * H + c], acc);
+        }
+        out[(size_t)t * H + c] = from_f32<TC>(acc);
+    }
+}
+
+extern "C" int spy_moe_combine(void* out, int dtype, const float* Y, const float* weights, const int* pair_row, int T, int top, int H,
+                               hipStream_t st) {
+    SPY_REQUIRE(T > 0 && top > 0 && H > 0, "spy_moe_combine: empty operand");
+    SPY_DISPATCH(dtype, TC, (moe_combine_kernel<TC><<<T, 256, 0, st>>>((TC*)out, Y, weights, pair_row, top, H)));
+    SPY_CHECK_LAUNCH("spy_moe_combine");
+    return 0;
+}

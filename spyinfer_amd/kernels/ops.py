@@ -76,7 +76,9 @@ class _Hip:
                      "spy_sample", "spy_sample_workspace", "spy_gemm_skinny", "spy_gemm_skinny_swiglu",
                      "spy_gemm_decode", "spy_gemm_decode_workspace", "spy_embedding_sumsq", "spy_sample_static", "spy_measure_read",
                      "spy_pair_embedding", "spy_norm_residual", "spy_depth_mix", "spy_xielu", "spy_mingru", "spy_latent_prepare",
-                     "spy_gemm_strided", "spy_latent_attention", "spy_latent_attention_mfma", "spy_latent_attention_mfma_workspace", "spy_head_products"):
+                     "spy_gemm_strided", "spy_latent_attention", "spy_latent_attention_mfma", "spy_latent_attention_mfma_workspace", "spy_head_products",
+                     "spy_bias_rope_store", "spy_sigmoid_gate", "spy_mlstm", "spy_causal_conv_silu", "spy_delta_rule", "spy_moe_route",
+                     "spy_moe_align", "spy_moe_gemm", "spy_moe_combine", "spy_moe_tile_rows"):
             if not hasattr(self.lib, name):
                 raise KernelError("the kernel library %s lacks %s: it is older than its sources; build it again "
                                   "(spyinfer_amd.kernels.build.build())" % (self.lib._name, name))
@@ -120,8 +122,8 @@ def library_path() -> str:
 
 
 # --------------------------------------------------------------------------
-def embedding(ids: torch.Tensor, table: torch.Tensor) -> torch.Tensor:
-    """out[t, :] = table[ids[t], :] widened to float32 (the start of the residual stream)."""
+def embedding(ids: torch.Tensor, table: torch.Tensor, scale: float = 1.0) -> torch.Tensor:
+    """out[t, :] = table[ids[t], :] * scale widened to float32 (the start of the residual stream)."""
     _dev(ids, table)
     _check(ids.dtype == torch.int32 and ids.dim() == 1, "embedding: ids must be int32 [T]")
     _check(table.dim() == 2, "embedding: table must be [V, H]")
@@ -129,18 +131,21 @@ def embedding(ids: torch.Tensor, table: torch.Tensor) -> torch.Tensor:
     out = torch.empty((T, H), dtype=torch.float32, device=table.device)
     if T:
         hip().call("spy_embedding", _ptr(out), _ptr(table), _code(table, "embedding table"), _ptr(ids),
-                   ctypes.c_int(T), ctypes.c_int(H), ctypes.c_int(V), _Hip.stream())
+                   ctypes.c_int(T), ctypes.c_int(H), ctypes.c_int(V), ctypes.c_float(scale), _Hip.stream())
     return out
 
 
 def add_rms_norm(resid: torch.Tensor, delta: Optional[torch.Tensor], weight: torch.Tensor, eps: float,
-                 out_dtype: torch.dtype, rows: Optional[torch.Tensor] = None) -> torch.Tensor:
-    """resid += delta (float32, in place; skipped if delta is None), then RMS-normalise.
+                 out_dtype: torch.dtype, rows: Optional[torch.Tensor] = None, delta2: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """resid += delta (float32, in place; skipped if delta is None), then RMS-normalise.  ``delta2``: a second addend
+    (two sublayers that read one norm): resid += delta + delta2, the two summed in float32 first.
 
     Without ``rows``: every row is updated and normalised -> [T, H].  With ``rows``
     (int32 [R]): only those rows are summed and normalised -> [R, H]; resid is left as it is."""
-    _dev(resid, delta, weight, rows)
+    _dev(resid, delta, weight, rows, delta2)
     _check(resid.dtype == torch.float32 and resid.dim() == 2, "add_rms_norm: the residual stream must be float32 [T, H]")
+    if delta2 is not None:
+        _check(delta is not None and delta2.shape == delta.shape and delta2.dtype == delta.dtype, "add_rms_norm: the second addend must be like the first")
     T, H = resid.shape
     _check(weight.shape == (H,), "add_rms_norm: weight must be [H]")
     if delta is not None:
@@ -150,7 +155,7 @@ def add_rms_norm(resid: torch.Tensor, delta: Optional[torch.Tensor], weight: tor
     n_out = T if rows is None else rows.shape[0]
     out = torch.empty((n_out, H), dtype=out_dtype, device=resid.device)
     if n_out:
-        hip().call("spy_add_rmsnorm", _ptr(resid), _ptr(delta), _ptr(weight), _code(weight, "norm weight"),
+        hip().call("spy_add_rmsnorm", _ptr(resid), _ptr(delta), _ptr(delta2), _ptr(weight), _code(weight, "norm weight"),
                    ctypes.c_float(eps), _ptr(out), _code(out, "norm output"), _ptr(rows), ctypes.c_int(n_out),
                    ctypes.c_int(T), ctypes.c_int(H), _Hip.stream())
     return out
@@ -1132,6 +1137,208 @@ def latent_attention(qa: torch.Tensor, cache: torch.Tensor, page_size: int, meta
                    ctypes.c_int(meta.max_blocks), _ptr(meta.token_entry), _ptr(meta.positions), _ptr(sink),
                    _code(sink, "sink") if sink is not None else F32, ctypes.c_int(meta.S), ctypes.c_int(T), ctypes.c_int(H),
                    ctypes.c_int(R), ctypes.c_int(D - R), ctypes.c_float(scale), ctypes.c_int(int(window or 0)), _Hip.stream())
+    return out
+
+
+# --------------------------------------------------------------------------
+# Attention layers with projection biases, heads rotated in part by angles formed in the kernel, and an output gate
+def _row_view(x: torch.Tensor, what: str) -> int:
+    """Rows of a wider product: a 2-D view on the GPU whose values lie side by side; returns the row stride."""
+    _check(x.is_cuda and x.dim() == 2 and x.stride(1) == 1 and x.dtype in _CODES, "%s: rows of float32 or bfloat16 on the GPU expected", what)
+    return x.stride(0)
+
+
+def bias_rope_store(x: torch.Tensor, n_q: int, n_kv: int, d: int, bias: Optional[torch.Tensor], freq: Optional[torch.Tensor],
+                    rotary_dim: int, positions: torch.Tensor, k_cache, v_cache, page_size: int, slots: Optional[torch.Tensor]) -> torch.Tensor:
+    """From rows ``x [T, >= (n_q + 2 n_kv) d]`` = [q heads | k heads | v heads] (a view into a wider product may be
+    given): the biases ``bias [(n_q + 2 n_kv) d]`` added, the first ``rotary_dim`` dims of every q and k head rotated
+    (pair (j, j + rotary_dim/2), angle float32(position) * freq[j]), q written to the result [T, n_q d], k and v into
+    the cache pages at ``slots`` (skipped when None)."""
+    xs = _row_view(x, "bias_rope_store")
+    T = x.shape[0]
+    _dev(bias, freq, positions, k_cache, v_cache, slots)
+    _check(x.shape[1] >= (n_q + 2 * n_kv) * d, "bias_rope_store: rows of %d values hold no %d heads of %d", x.shape[1], n_q + 2 * n_kv, d)
+    _check(bias is None or bias.shape == ((n_q + 2 * n_kv) * d,), "bias_rope_store: one bias per projected value expected")
+    _check(positions.dtype == torch.int32 and positions.shape == (T,), "bias_rope_store: positions must be int32 [T]")
+    _check(rotary_dim == 0 or (freq is not None and freq.dtype == torch.float32 and freq.shape == (rotary_dim // 2,) and rotary_dim % 2 == 0
+                               and rotary_dim <= d), "bias_rope_store: one float32 frequency per rotated pair expected")
+    num_pages = 0
+    if slots is not None:
+        _check(slots.dtype == torch.int32 and slots.shape == (T,), "bias_rope_store: slots must be int32 [T]")
+        num_pages = k_cache.shape[0]
+        _check(k_cache.dtype == x.dtype and v_cache.dtype == x.dtype and tuple(k_cache.shape) == (num_pages, n_kv, page_size, d)
+               and tuple(v_cache.shape) == (num_pages, n_kv, d, page_size),
+               "bias_rope_store: cache pages must be K [pages, n_kv, page, d] and V [pages, n_kv, d, page] of the activation dtype")
+    q = torch.empty((T, n_q * d), dtype=x.dtype, device=x.device)
+    if T:
+        hip().call("spy_bias_rope_store", ctypes.c_void_p(x.data_ptr()), ctypes.c_longlong(xs), _code(x, "x"), _ptr(q), ctypes.c_int(T),
+                   ctypes.c_int(n_q), ctypes.c_int(n_kv), ctypes.c_int(d), _ptr(bias), _code(bias, "bias") if bias is not None else F32,
+                   _ptr(freq), ctypes.c_int(rotary_dim), _ptr(positions), _ptr(k_cache if slots is not None else None),
+                   _ptr(v_cache if slots is not None else None), ctypes.c_int(page_size), ctypes.c_int(num_pages), _ptr(slots), _Hip.stream())
+    return q
+
+
+def sigmoid_gate(y: torch.Tensor, gate: torch.Tensor) -> torch.Tensor:
+    """In place: y[t, j] *= sigmoid(gate[t, j]); ``gate`` may be a view into a wider product."""
+    _dev(y)
+    gs = _row_view(gate, "sigmoid_gate")
+    _check(y.dim() == 2 and gate.shape == y.shape and gate.dtype == y.dtype and gate.device == y.device, "sigmoid_gate: gate rows like y expected")
+    if y.numel():
+        hip().call("spy_sigmoid_gate", _ptr(y), ctypes.c_void_p(gate.data_ptr()), ctypes.c_longlong(gs), _code(y, "y"), ctypes.c_int(y.shape[0]),
+                   ctypes.c_int(y.shape[1]), _Hip.stream())
+    return y
+
+
+# --------------------------------------------------------------------------
+# Recurrent mixers with a matrix state per head
+MATRIX_MEMORY_MAX_DIM, MATRIX_MEMORY_MAX_VDIM = 256, 1024
+
+
+def _entries(cu_q: torch.Tensor, slot_ids: torch.Tensor, what: str) -> int:
+    S = slot_ids.shape[0]
+    _check(cu_q.dtype == torch.int32 and cu_q.shape == (S + 1,) and slot_ids.dtype == torch.int32, "%s: cu_q int32 [S + 1] and slot_ids int32 [S] expected", what)
+    return S
+
+
+def mlstm(x: torch.Tensor, q_off: int, k_off: int, v_off: int, g_off: int, gates: torch.Tensor, bi: torch.Tensor, bf: torch.Tensor,
+          cap: float, norm_w: torch.Tensor, eps: float, state: torch.Tensor, cu_q: torch.Tensor, slot_ids: torch.Tensor, H: int, d: int,
+          dv: int) -> torch.Tensor:
+    """The mLSTM recurrence over the step's tokens.  ``x``: rows of the fused projection with q (H heads of d) at column
+    ``q_off``, k at ``k_off``, v (H heads of dv) at ``v_off`` and the output gate's rows at ``g_off``; ``gates [T, 2 H]``
+    float32: the raw products of the input and forget gates (their biases ``bi``, ``bf [H]``; both capped by
+    cap tanh(. / cap)); ``state [slots, H (d dv + d + 1)]`` float32 holds S, n and the running maximum of every head, read
+    at an entry's start and left at its end.  Returns [T, H dv]: each head's read-out over its root mean square, times
+    ``norm_w``, times sigmoid(gate)."""
+    xs = _row_view(x, "mlstm")
+    T = x.shape[0]
+    _dev(gates, bi, bf, norm_w, state, cu_q, slot_ids)
+    S = _entries(cu_q, slot_ids, "mlstm")
+    _check(0 < d <= MATRIX_MEMORY_MAX_DIM and 0 < dv <= MATRIX_MEMORY_MAX_VDIM, "mlstm: heads of %d x %d (up to %d x %d)", d, dv,
+           MATRIX_MEMORY_MAX_DIM, MATRIX_MEMORY_MAX_VDIM)
+    _check(max(q_off, k_off) + H * d <= x.shape[1] and max(v_off, g_off) + H * dv <= x.shape[1] and min(q_off, k_off, v_off, g_off) >= 0,
+           "mlstm: the projections' columns reach beyond the rows")
+    _check(gates.dtype == torch.float32 and gates.shape == (T, 2 * H), "mlstm: the gates' products must be float32 [T, 2 H]")
+    _check(bi.shape == (H,) and bf.shape == (H,) and norm_w.shape == (H * dv,) and bi.dtype == bf.dtype == norm_w.dtype,
+           "mlstm: gate biases [H] and a norm weight [H dv] of one dtype expected")
+    _check(state.dtype == torch.float32 and state.dim() == 2 and state.shape[1] == H * (d * dv + d + 1), "mlstm: state must be float32 [slots, H (d dv + d + 1)]")
+    out = torch.empty((T, H * dv), dtype=x.dtype, device=x.device)
+    if T:
+        hip().call("spy_mlstm", _ptr(out), _ptr(state), ctypes.c_void_p(x.data_ptr()), ctypes.c_longlong(xs), _code(x, "x"), ctypes.c_int(q_off),
+                   ctypes.c_int(k_off), ctypes.c_int(v_off), ctypes.c_int(g_off), _ptr(gates), _ptr(bi), _ptr(bf), _code(bi, "gate biases"),
+                   ctypes.c_float(cap), _ptr(norm_w), ctypes.c_float(eps), _ptr(cu_q), _ptr(slot_ids), ctypes.c_int(state.shape[0]),
+                   ctypes.c_int(S), ctypes.c_int(T), ctypes.c_int(H), ctypes.c_int(d), ctypes.c_int(dv), _Hip.stream())
+    return out
+
+
+def causal_conv_silu(x: torch.Tensor, taps: torch.Tensor, state: torch.Tensor, keep_off: int, token_entry: torch.Tensor,
+                     cu_q: torch.Tensor, slot_ids: torch.Tensor) -> torch.Tensor:
+    """y[t, c] = silu(sum_j taps[c, j] x[t - (n - 1) + j, c]) per request (``x [T, C]`` may be a view into a wider
+    product); inputs before an entry's first token are the request's kept inputs ``state[slot, keep_off + i C + c]``
+    (i = 0 .. n - 2, the newest last; float32), which afterwards hold the entry's last n - 1 inputs."""
+    xs = _row_view(x, "causal_conv_silu")
+    T, C = x.shape
+    _dev(taps, state, token_entry, cu_q, slot_ids)
+    S = _entries(cu_q, slot_ids, "causal_conv_silu")
+    _check(taps.dim() == 2 and taps.shape[0] == C and 1 <= taps.shape[1] <= 8, "causal_conv_silu: taps [C, 1..8] expected")
+    n = taps.shape[1]
+    _check(token_entry.dtype == torch.int32 and token_entry.shape == (T,), "causal_conv_silu: token_entry must be int32 [T]")
+    _check(state.dtype == torch.float32 and state.dim() == 2 and 0 <= keep_off and keep_off + (n - 1) * C <= state.shape[1],
+           "causal_conv_silu: the kept inputs reach beyond the float32 state")
+    y = torch.empty((T, C), dtype=x.dtype, device=x.device)
+    if T:
+        hip().call("spy_causal_conv_silu", _ptr(y), ctypes.c_void_p(x.data_ptr()), ctypes.c_longlong(xs), _code(x, "x"), _ptr(taps),
+                   _code(taps, "taps"), ctypes.c_void_p(state.data_ptr() + 4 * keep_off), ctypes.c_longlong(state.shape[1]), _ptr(token_entry),
+                   _ptr(cu_q), _ptr(slot_ids), ctypes.c_int(state.shape[0]), ctypes.c_int(S), ctypes.c_int(T), ctypes.c_int(C), ctypes.c_int(n),
+                   _Hip.stream())
+    return y
+
+
+def delta_rule(qkv: torch.Tensor, beta_pre: torch.Tensor, dec_pre: torch.Tensor, a_log: torch.Tensor, dt_bias: torch.Tensor,
+               gate: torch.Tensor, norm_w: torch.Tensor, eps: float, state: torch.Tensor, cu_q: torch.Tensor, slot_ids: torch.Tensor,
+               H: int, G: int, d: int, dv: int) -> torch.Tensor:
+    """The gated delta rule over the step's tokens.  ``qkv [T, 2 G d + H dv]``: q and k (G heads of d; made unit vectors
+    here, q also times d^-1/2) and v (H heads of dv); ``beta_pre [T, H]`` and ``dec_pre [T, H d]`` float32: the raw products
+    behind beta = sigmoid(.) and the decay exp(-exp(a_log[h]) softplus(. + dt_bias)) per head and key channel; per head
+    S = diag(decay) S, u = beta (v - S^T k), S += k u^T, o = S^T q with ``state[slot, h d dv ..]`` float32.  Returns
+    [T, H dv]: o over its root mean square, times ``norm_w [dv]``, times sigmoid(``gate``) (rows of H dv values, a view
+    into a wider product allowed)."""
+    _dev(qkv, beta_pre, dec_pre, a_log, dt_bias, norm_w, state, cu_q, slot_ids)
+    gs = _row_view(gate, "delta_rule")
+    T = qkv.shape[0]
+    S = _entries(cu_q, slot_ids, "delta_rule")
+    _check(qkv.dim() == 2 and qkv.shape[1] == 2 * G * d + H * dv and qkv.dtype in _CODES and gate.dtype == qkv.dtype and gate.shape == (T, H * dv),
+           "delta_rule: qkv [T, 2 G d + H dv] and gate rows [T, H dv] of one dtype expected")
+    _check(H % G == 0 and 0 < d <= MATRIX_MEMORY_MAX_DIM and 0 < dv <= MATRIX_MEMORY_MAX_VDIM, "delta_rule: heads of %d x %d (up to %d x %d)",
+           d, dv, MATRIX_MEMORY_MAX_DIM, MATRIX_MEMORY_MAX_VDIM)
+    _check(beta_pre.dtype == torch.float32 and beta_pre.shape == (T, H) and dec_pre.dtype == torch.float32 and dec_pre.shape == (T, H * d),
+           "delta_rule: the products behind beta [T, H] and the decay [T, H d] must be float32")
+    _check(a_log.shape == (H,) and dt_bias.shape == (H * d,) and norm_w.shape == (dv,) and a_log.dtype == dt_bias.dtype == norm_w.dtype,
+           "delta_rule: a_log [H], dt_bias [H d] and a norm weight [dv] of one dtype expected")
+    _check(state.dtype == torch.float32 and state.dim() == 2 and state.shape[1] >= H * d * dv, "delta_rule: state must be float32 [slots, >= H d dv]")
+    out = torch.empty((T, H * dv), dtype=qkv.dtype, device=qkv.device)
+    if T:
+        hip().call("spy_delta_rule", _ptr(out), _ptr(state), ctypes.c_longlong(state.shape[1]), _ptr(qkv), _code(qkv, "qkv"), _ptr(beta_pre),
+                   _ptr(dec_pre), _ptr(a_log), _ptr(dt_bias), _code(a_log, "decay numbers"), ctypes.c_void_p(gate.data_ptr()), ctypes.c_longlong(gs),
+                   _ptr(norm_w), ctypes.c_float(eps), _ptr(cu_q), _ptr(slot_ids), ctypes.c_int(state.shape[0]), ctypes.c_int(S), ctypes.c_int(T),
+                   ctypes.c_int(H), ctypes.c_int(G), ctypes.c_int(d), ctypes.c_int(dv), _Hip.stream())
+    return out
+
+
+# --------------------------------------------------------------------------
+# Mixture of experts
+def moe_route(z: torch.Tensor, correction: torch.Tensor, top: int, groups: int, keep: int, scale: float):
+    """Router logits ``z [T, E]`` float32 -> (experts int32 [T, top], weights float32 [T, top]): s = softmax(z); the choice
+    goes by s + ``correction`` among the experts of the ``keep`` best of ``groups`` equal groups of neighbours (a group's
+    score: its largest choice score); the weights are the chosen s over their sum (+ 1e-20), times ``scale``."""
+    _dev(z, correction)
+    _check(z.dtype == torch.float32 and z.dim() == 2 and correction.dtype == torch.float32 and correction.shape == (z.shape[1],),
+           "moe_route: logits float32 [T, E] and a float32 correction [E] expected")
+    T, E = z.shape
+    _check(0 < groups and E % groups == 0 and 0 < keep <= groups and 0 < top <= keep * (E // groups) and E <= 1024,
+           "moe_route: %d choices among %d of %d groups of %d experts" % (top, keep, groups, E))
+    ids = torch.empty((T, top), dtype=torch.int32, device=z.device)
+    w = torch.empty((T, top), dtype=torch.float32, device=z.device)
+    if T:
+        hip().call("spy_moe_route", _ptr(ids), _ptr(w), _ptr(z), _ptr(correction), ctypes.c_int(T), ctypes.c_int(E), ctypes.c_int(top),
+                   ctypes.c_int(groups), ctypes.c_int(keep), ctypes.c_float(scale), _Hip.stream())
+    return ids, w
+
+
+def moe_experts(x: torch.Tensor, ids: torch.Tensor, weights: torch.Tensor, w_gate_up: torch.Tensor, w_down: torch.Tensor) -> torch.Tensor:
+    """out[t] = sum_k weights[t, k] * down_e( silu(gate_e x[t]) * up_e x[t] ), e = ids[t, k]; ``w_gate_up [E, 2 F, K]`` =
+    every expert's [gate rows | up rows], ``w_down [E, K, F]``.  The (token, choice) pairs are sorted by expert on the
+    device and the experts' products run over the sorted rows; no size here depends on the choice."""
+    _dev(x, ids, weights, w_gate_up, w_down)
+    T, K = x.shape
+    top = ids.shape[1]
+    E, F2, _ = w_gate_up.shape
+    F = F2 // 2
+    _check(x.dim() == 2 and ids.dtype == torch.int32 and ids.shape == (T, top) and weights.dtype == torch.float32 and weights.shape == (T, top),
+           "moe_experts: experts int32 [T, top] and weights float32 [T, top] expected")
+    _check(w_gate_up.dim() == 3 and w_gate_up.shape == (E, 2 * F, K) and tuple(w_down.shape) == (E, K, F) and w_down.dtype == w_gate_up.dtype,
+           "moe_experts: expert matrices [E, 2 F, K] and [E, K, F] of one dtype expected")
+    out = torch.empty((T, K), dtype=x.dtype, device=x.device)
+    if not T:
+        return out
+    tm = hip().lib.spy_moe_tile_rows()
+    P = T * top
+    max_tiles = P // tm + min(E, P)
+    dev = x.device
+    sorted_pair = torch.empty((max_tiles * tm,), dtype=torch.int32, device=dev)
+    pair_row = torch.empty((P,), dtype=torch.int32, device=dev)
+    tile_expert = torch.empty((max_tiles,), dtype=torch.int32, device=dev)
+    hip().call("spy_moe_align", _ptr(sorted_pair), _ptr(pair_row), _ptr(tile_expert), _ptr(ids), ctypes.c_int(P), ctypes.c_int(E),
+               ctypes.c_int(max_tiles), _Hip.stream())
+    act = torch.empty((max_tiles * tm, F), dtype=x.dtype, device=dev)
+    hip().call("spy_moe_gemm", _ptr(act), _code(act, "act"), _ptr(x), _code(x, "x"), _ptr(w_gate_up), _code(w_gate_up, "expert matrices"),
+               _ptr(tile_expert), _ptr(sorted_pair), ctypes.c_int(top), ctypes.c_int(1), ctypes.c_int(max_tiles), ctypes.c_int(E), ctypes.c_int(F),
+               ctypes.c_int(K), _Hip.stream())
+    y = torch.empty((max_tiles * tm, K), dtype=torch.float32, device=dev)
+    hip().call("spy_moe_gemm", _ptr(y), F32, _ptr(act), _code(act, "act"), _ptr(w_down), _code(w_down, "expert matrices"), _ptr(tile_expert),
+               _ptr(sorted_pair), ctypes.c_int(0), ctypes.c_int(0), ctypes.c_int(max_tiles), ctypes.c_int(E), ctypes.c_int(K), ctypes.c_int(F),
+               _Hip.stream())
+    hip().call("spy_moe_combine", _ptr(out), _code(out, "out"), _ptr(y), _ptr(weights), _ptr(pair_row), ctypes.c_int(T), ctypes.c_int(top),
+               ctypes.c_int(K), _Hip.stream())
     return out
 
 

@@ -1,3 +1,4 @@
 from . import qwen3  # registers "Qwen3ForCausalLM"
 from . import sefevik  # registers "Sefevik"
+from . import sodedra  # registers "Sodedra"
 from .base import DecoderModel, LayerCall

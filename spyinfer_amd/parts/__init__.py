@@ -1,9 +1,9 @@
 from .attention import PagedAttention
 from .base import Block, FeedForward, Mixer, Norm, Part, PositionEncoding
-from .block import DepthMix, OutputNormBlock, PreNormBlock
+from .block import DepthMix, OutputNormBlock, ParallelBlock, PreNormBlock
 from .embedding import LMHead, PairHashEmbedding, TokenEmbedding
 from .latent_attention import LatentAttention
-from .mlp import DenseMLP, GatedMLP
+from .mlp import DenseMLP, GatedMLP, MoEMLP
 from .norm import RMSNorm
-from .recurrent import MinGRU
+from .recurrent import ChannelDelta, MinGRU, MLSTM
 from .rotary import RotaryEmbedding

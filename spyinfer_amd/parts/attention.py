@@ -8,6 +8,12 @@ through its request's block table with the causal mask ``key <= position``
 (:98-111), scale 1/sqrt(d) after the dot product (:59, :110), kv head
 ``h * n_kv / n_q`` (:96); output projection.  One meaning for whole prompts,
 portions and single tokens.  ``window`` keeps only the last ``window`` keys.
+
+Options beside the reference's arrangement: biases on the q, k and v projections; a value size other than the
+key size (the smaller of the two is padded with zero rows when the weights are bound, so that one head size runs
+through cache and kernels); a sigmoid gate on the concatenated heads, projected from the mixer's input beside
+q, k and v; a rotation whose angles are formed in the kernel from the encoding's frequencies (no table and no
+position limit: encodings with rescaled frequencies).
 """
 from __future__ import annotations
 
@@ -95,12 +101,24 @@ def attention_meta(batch, group: int, group_size: int, big_rows: int = 0) -> ops
 class PagedAttention(Mixer):
     def __init__(self, hidden_size: int, num_heads: int, num_kv_heads: int, head_dim: int,
                  position: Optional[PositionEncoding], qk_norm_eps: Optional[float] = None,
-                 window: Optional[int] = None, scale: Optional[float] = None, fold_rows: Optional[int] = None):
+                 window: Optional[int] = None, scale: Optional[float] = None, fold_rows: Optional[int] = None,
+                 value_dim: Optional[int] = None, bias: bool = False, gate: bool = False, names: Optional[dict] = None):
         """``fold_rows``: most rows of a step whose products here run with the norms and the residual sum folded in
-        (None: ``ops.default_fold_rows`` of this part's matrices)."""
+        (None: ``ops.default_fold_rows`` of this part's matrices).  ``value_dim``: size of a value head (None: ``head_dim``).
+        ``bias``: q, k and v have biases.  ``gate``: the heads' results are multiplied by sigmoid(Wg x) before the output
+        projection.  ``names``: tensor names behind the prefix for q, k, v, o, g, q_norm, k_norm and the biases' suffix
+        ``bias``."""
         if num_heads % num_kv_heads:
             raise ValueError("num_heads must be a multiple of num_kv_heads")
-        self.hidden_size, self.num_heads, self.num_kv_heads, self.head_dim = hidden_size, num_heads, num_kv_heads, head_dim
+        self.hidden_size, self.num_heads, self.num_kv_heads = hidden_size, num_heads, num_kv_heads
+        self.key_dim, self.value_dim = head_dim, head_dim if value_dim is None else value_dim
+        # one head size for cache and kernels: where key and value sizes differ, the larger, in whole MFMA tiles
+        self.head_dim = head_dim if self.value_dim == head_dim else -(-max(head_dim, self.value_dim) // 16) * 16
+        self.has_bias, self.has_gate = bool(bias), bool(gate)
+        self.names = dict(q=".q_proj.weight", k=".k_proj.weight", v=".v_proj.weight", o=".o_proj.weight", g=".g_proj.weight",
+                          q_norm=".q_norm.weight", k_norm=".k_norm.weight", bias=".bias")
+        self.names.update(names or {})
+        self.b_qkv = None
         self.position = position
         self.qk_norm_eps = qk_norm_eps
         self.window = window
@@ -110,28 +128,56 @@ class PagedAttention(Mixer):
 
     # ---- weights ---------------------------------------------------------
     def weight_specs(self, prefix):
-        H, nq, nkv, d = self.hidden_size, self.num_heads, self.num_kv_heads, self.head_dim
-        specs = [WeightSpec(prefix + ".q_proj.weight", (nq * d, H)), WeightSpec(prefix + ".k_proj.weight", (nkv * d, H)),
-                 WeightSpec(prefix + ".v_proj.weight", (nkv * d, H)), WeightSpec(prefix + ".o_proj.weight", (H, nq * d))]
+        H, nq, nkv, dk, dv, n = self.hidden_size, self.num_heads, self.num_kv_heads, self.key_dim, self.value_dim, self.names
+        specs = [WeightSpec(prefix + n["q"], (nq * dk, H)), WeightSpec(prefix + n["k"], (nkv * dk, H)),
+                 WeightSpec(prefix + n["v"], (nkv * dv, H)), WeightSpec(prefix + n["o"], (H, nq * dv))]
+        if self.has_bias:
+            specs += [WeightSpec(prefix + n["q"] + n["bias"], (nq * dk,), "bias"), WeightSpec(prefix + n["k"] + n["bias"], (nkv * dk,), "bias"),
+                      WeightSpec(prefix + n["v"] + n["bias"], (nkv * dv,), "bias")]
+        if self.has_gate:
+            specs.append(WeightSpec(prefix + n["g"], (nq * dv, H)))
         if self.qk_norm_eps is not None:
-            specs += [WeightSpec(prefix + ".q_norm.weight", (d,), "norm"), WeightSpec(prefix + ".k_norm.weight", (d,), "norm")]
+            specs += [WeightSpec(prefix + n["q_norm"], (dk,), "norm"), WeightSpec(prefix + n["k_norm"], (dk,), "norm")]
         return specs
 
+    def _padded(self, t: torch.Tensor, heads: int, size: int) -> torch.Tensor:
+        """Rows (or entries) [heads * size, ...] -> [heads * head_dim, ...], every head filled up with zeros."""
+        d = self.head_dim
+        if size == d:
+            return t
+        out = torch.zeros((heads, d) + tuple(t.shape[1:]), dtype=t.dtype, device=t.device)
+        out[:, :size] = t.view((heads, size) + tuple(t.shape[1:]))
+        return out.view((heads * d,) + tuple(t.shape[1:]))
+
     def bind(self, prefix, weights):
-        # the three matrices leave the caller's dictionary here, so that they are freed once they are fused: binding a
+        # the matrices leave the caller's dictionary here, so that they are freed once they are fused: binding a
         # model never holds the separate matrices, the fused one and its tiled copy of all layers at once
-        q, k, v = (weights.pop(prefix + ".%s_proj.weight" % n) for n in "qkv")
-        if not (q.dtype == k.dtype == v.dtype):
-            q, k, v = q.float(), k.float(), v.float()
-        # one product for q, k and v: rows [q heads | k heads | v heads]
-        self.w_qkv = torch.cat([q, k, v], dim=0).contiguous()
-        del q, k, v
+        n, nq, nkv, dk, dv = self.names, self.num_heads, self.num_kv_heads, self.key_dim, self.value_dim
+        mats = [weights.pop(prefix + n[c]) for c in "qkv"] + ([weights.pop(prefix + n["g"])] if self.has_gate else [])
+        if len({m.dtype for m in mats}) > 1:
+            mats = [m.float() for m in mats]
+        mats = [self._padded(m, heads, size) for m, heads, size in zip(mats, (nq, nkv, nkv, nq), (dk, dk, dv, dv))]
+        # one product for q, k and v (and the gate): rows [q heads | k heads | v heads | gate]
+        self.w_qkv = torch.cat(mats, dim=0).contiguous()
+        del mats
         self.w_qkv, self.w_qkv_tiled = ops.weight_forms(self.w_qkv)
-        self.w_o, self.w_o_tiled = ops.weight_forms(weights.pop(prefix + ".o_proj.weight"))
+        w_o = weights.pop(prefix + n["o"])
+        if dv != self.head_dim:
+            w_o = self._padded(w_o.t().contiguous(), nq, dv).t().contiguous()
+        self.w_o, self.w_o_tiled = ops.weight_forms(w_o)
+        if self.has_bias:
+            b = [weights[prefix + n[c] + n["bias"]] for c in "qkv"]
+            if len({t.dtype for t in b}) > 1:
+                b = [t.float() for t in b]
+            self.b_qkv = torch.cat([self._padded(t, heads, size) for t, heads, size in zip(b, (nq, nkv, nkv), (dk, dk, dv))]).contiguous()
         if self.qk_norm_eps is not None:
-            self.q_norm, self.k_norm = weights[prefix + ".q_norm.weight"], weights[prefix + ".k_norm.weight"]
+            if dk != self.head_dim:
+                raise ValueError("per-head norms of q and k with a value size other than the key size are not implemented")
+            self.q_norm, self.k_norm = weights[prefix + n["q_norm"]], weights[prefix + n["k_norm"]]
             if self.q_norm.dtype != self.k_norm.dtype:
                 self.q_norm, self.k_norm = self.q_norm.float(), self.k_norm.float()
+        if self.position is not None and not self._plain_projections():
+            self.position.prepare(self.w_o.device, 0)
 
     # ---- cache -----------------------------------------------------------
     def cache_spec(self):
@@ -152,8 +198,16 @@ class PagedAttention(Mixer):
                 key_pieces.decode_pieces_capacity(entries, self.num_kv_heads) * key_pieces.PIECE_RECORD
         return out
 
+    def _plain_projections(self) -> bool:
+        """No bias, no gate and a rotation by table: the arrangement that the fused kernels and the folded products know.
+        Otherwise one kernel adds the biases, rotates by angles that it forms itself from the encoding's frequencies (an
+        encoding with rescaled frequencies has no table) and stores."""
+        return not (self.has_bias or self.has_gate or (self.position is not None and getattr(self.position, "scaling", None) is not None))
+
     def _rotated_whole(self) -> bool:
         """The head is rotated whole or not at all, and the group is one tile: what the fused kernel takes."""
+        if not self._plain_projections():
+            return False
         rot = self.position.rotary() if self.position is not None else None
         return (rot is None or rot[2] in (0, self.head_dim)) and self.num_heads // self.num_kv_heads <= 16
 
@@ -176,6 +230,8 @@ class PagedAttention(Mixer):
 
     def can_fold(self, batch):
         # (beyond 64 rows the products take their inputs in operand order only: the attention must hand its result over so)
+        if not self._plain_projections():
+            return False
         if batch.T > 64 and not ops.attention_hands_over_operand_rows(batch.act_dtype, self.num_heads, self.head_dim, batch.page_size):
             return False
         return ops.fused_decode_ok(batch.T, batch.act_dtype, self.w_qkv_tiled, self.w_o_tiled, max_rows=self.fold_rows)
@@ -186,10 +242,26 @@ class PagedAttention(Mixer):
             qkv = ops.decode_linear(x, self.w_qkv_tiled)
         else:
             qkv = ops.linear(x, self.w_qkv, tiled=self.w_qkv_tiled)
+        meta = attention_meta(batch, cache.group, nq // nkv, self._big_rows(batch, cache.page_size))
+        if not self._plain_projections():
+            # biases, rotation and store in one kernel that reads q, k and v out of the wider product; the gate's rows,
+            # which lie behind them, are multiplied into the heads' results
+            if self.qk_norm_eps is not None:
+                raise ValueError("per-head norms of q and k beside biases, a gate or rescaled frequencies are not implemented")
+            freq, rdim = None, 0
+            if self.position is not None:
+                freq, mag, rdim = self.position.frequencies()
+                if mag != 1.0:
+                    raise ValueError("a factor on cos and sin is not implemented for this attention")
+            slots = batch.slot_mapping(cache.group) if store else None
+            q = ops.bias_rope_store(qkv, nq, nkv, d, self.b_qkv, freq, rdim, batch.positions, cache.k, cache.v, cache.page_size, slots)
+            out = ops.paged_attention(q, cache.k, cache.v, cache.page_size, meta, nq, nkv, d, self.scale, self.window)
+            if self.has_gate:
+                ops.sigmoid_gate(out, qkv[:, (nq + 2 * nkv) * d:])
+            return out
         rot = self.position.rotary() if self.position is not None else None
         cos, sin, rdim = rot if rot is not None else (None, None, 0)
         eps = self.qk_norm_eps if self.qk_norm_eps is not None else 0.0
-        meta = attention_meta(batch, cache.group, nq // nkv, self._big_rows(batch, cache.page_size))
         if ops.fused_attention_ok(qkv.dtype, meta, nq, nkv, d, cache.page_size, rdim, self.q_norm, self.k_norm):
             # single tokens only: the attention kernel norms, rotates and stores by itself
             raw = ops.RawQKV(qkv, self.q_norm, self.k_norm, eps, cos if rdim else None, sin if rdim else None, store)

@@ -133,7 +133,7 @@ class Block(Part):
 
     def forward(self, resid: torch.Tensor, delta, batch, cache, store: bool = True, next_norm: Optional[Norm] = None):
         """(residual stream, pending) -> (residual stream, pending).  ``pending`` is None, an addend [T, H] that
-        the next norm sums into the stream, or a ``ScaledInput``: then the stream is complete and the input of
+        the next norm sums into the stream (or a pair of addends, from a block whose two sublayers read one norm), or a ``ScaledInput``: then the stream is complete and the input of
         the norm named in it is prepared (a block that cannot use it ignores it).  ``next_norm``: the norm that
         reads the stream after this block, if the caller knows it; only then may a ``ScaledInput`` be returned."""
         raise NotImplementedError

@@ -145,7 +145,8 @@ class OutputNormBlock(Block):
     def forward(self, resid, pending, batch, cache, store=True, next_norm=None):
         act = batch.act_dtype
         if pending is not None and not isinstance(pending, ops.ScaledInput):
-            resid.add_(pending.float())            # a block of another arrangement left an addend
+            for addend in (pending if isinstance(pending, (tuple, list)) else (pending,)):
+                resid.add_(addend.float())         # a block of another arrangement left an addend (or a pair of them)
         x = stream_copy(batch, resid)
         y = self.mixer.forward(x, batch, cache, store)
         out = self.depth.result_slot(batch, resid) if self.depth is not None else resid
@@ -158,3 +159,35 @@ class OutputNormBlock(Block):
             out, copy = self.norm2.add_normed(out, f, out, act, mix)
         stream_copy(batch, out, copy)
         return out, None
+
+
+class ParallelBlock(Block):
+    """h += mixer(n) + ffn(n) with n = norm(h): one norm, both sublayers read its output, and their results meet the
+    stream together.  The two results go on as a pair of addends, which the next norm's kernel sums in float32 and adds
+    to the stream in the pass that it makes anyway.  ``ffn`` may be absent."""
+
+    def __init__(self, norm: Norm, mixer: Mixer, ffn: FeedForward = None, names=("norm1", "mix", "mlp")):
+        self.norm, self.mixer, self.ffn = norm, mixer, ffn
+        self.names = names
+
+    def _parts(self, prefix):
+        parts = zip((self.norm, self.mixer, self.ffn), (prefix + "." + n for n in self.names))
+        return [(part, p) for part, p in parts if part is not None]
+
+    def weight_specs(self, prefix):
+        return [s for part, p in self._parts(prefix) for s in part.weight_specs(p)]
+
+    def bind(self, prefix, weights):
+        for part, p in self._parts(prefix):
+            part.bind(p, weights)
+
+    def capturable(self, batch):
+        return all(part.capturable(batch) for part, _ in self._parts(""))
+
+    def forward(self, resid, pending, batch, cache, store=True, next_norm=None):
+        act = batch.act_dtype
+        n = self.norm.add_norm(resid, None if isinstance(pending, ops.ScaledInput) else pending, act)
+        a = self.mixer.forward(n, batch, cache, store)
+        if self.ffn is None:
+            return resid, a
+        return resid, (a, self.ffn.forward(n, batch))

@@ -11,27 +11,29 @@ from .base import Part
 
 
 class TokenEmbedding(Part):
-    def __init__(self, vocab_size: int, hidden_size: int):
+    def __init__(self, vocab_size: int, hidden_size: int, scale: float = 1.0, suffix: str = ".weight"):
+        """``scale``: h[t] = E[id[t]] * scale (a tied head still reads the table as it is stored)."""
         self.vocab_size, self.hidden_size = vocab_size, hidden_size
+        self.scale, self.suffix = float(scale), suffix
         self.weight = None
 
     def weight_specs(self, prefix):
-        return [WeightSpec(prefix + ".weight", (self.vocab_size, self.hidden_size))]
+        return [WeightSpec(prefix + self.suffix, (self.vocab_size, self.hidden_size))]
 
     def bind(self, prefix, weights):
-        self.weight = weights[prefix + ".weight"]
+        self.weight = weights[prefix + self.suffix]
 
     def capturable(self, batch):
         return True
 
     def forward(self, ids):
-        return ops.embedding(ids, self.weight)
+        return ops.embedding(ids, self.weight, self.scale)
 
     def forward_for(self, ids, norm, act_dtype):
         """(stream, pending) with the input of ``norm`` prepared where few rows and a foldable norm allow it."""
         fold = norm.foldable(act_dtype) if norm is not None else None
-        if fold is None or not ops.fused_decode_ok(ids.shape[0], act_dtype):
-            return ops.embedding(ids, self.weight), None
+        if fold is None or self.scale != 1.0 or not ops.fused_decode_ok(ids.shape[0], act_dtype):
+            return ops.embedding(ids, self.weight, self.scale), None
         return ops.embedding_scaled(ids, self.weight, fold[0], fold[1], norm)
 
 

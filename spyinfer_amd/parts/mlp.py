@@ -1,6 +1,10 @@
 """Gated feed-forward: down( silu(gate(x)) * up(x) ), no biases
 (src/models/qwen3.hpp:232-263; src/backends/cpu/x64/kernels.cpp:242-247).
-Gate and up run as one product with rows [gate | up]."""
+Gate and up run as one product with rows [gate | up].
+
+``MoEMLP``: a mixture of such gated layers.  A router (float32) scores all experts, s = softmax(W_r x); the choice goes
+by s plus a stored correction, among the experts of the best groups of neighbouring experts only; a token's result is
+the sum of its chosen experts' results, weighted with the chosen s over their sum, times a constant."""
 from __future__ import annotations
 
 import torch
@@ -11,23 +15,26 @@ from .base import FeedForward
 
 
 class GatedMLP(FeedForward):
-    def __init__(self, hidden_size: int, intermediate_size: int, activation: str = "silu", fold_rows=None):
+    def __init__(self, hidden_size: int, intermediate_size: int, activation: str = "silu", fold_rows=None,
+                 names=(".gate_proj.weight", ".up_proj.weight", ".down_proj.weight")):
         """``fold_rows``: most rows of a step whose products here run with the norms and the residual sum folded in
-        (None: ``ops.default_fold_rows`` of this part's matrices)."""
+        (None: ``ops.default_fold_rows`` of this part's matrices).  ``names``: the tensors' names behind the prefix."""
         if activation != "silu":
             raise ValueError("GatedMLP: activation %r is not implemented" % activation)
         self.hidden_size, self.intermediate_size = hidden_size, intermediate_size
         self.fold_rows = fold_rows
+        self.names = names
         self.w_gate_up = self.w_down = self.w_gate_up_tiled = self.w_down_tiled = None
 
     def weight_specs(self, prefix):
         H, I = self.hidden_size, self.intermediate_size
-        return [WeightSpec(prefix + ".gate_proj.weight", (I, H)), WeightSpec(prefix + ".up_proj.weight", (I, H)),
-                WeightSpec(prefix + ".down_proj.weight", (H, I))]
+        gate, up, down = (prefix + n for n in self.names)
+        return [WeightSpec(gate, (I, H)), WeightSpec(up, (I, H)), WeightSpec(down, (H, I))]
 
     def bind(self, prefix, weights):
         # (popped: the separate matrices are freed once they are fused, see PagedAttention.bind)
-        g, u = weights.pop(prefix + ".gate_proj.weight"), weights.pop(prefix + ".up_proj.weight")
+        gate, up, down = (prefix + n for n in self.names)
+        g, u = weights.pop(gate), weights.pop(up)
         if g.dtype != u.dtype:
             g, u = g.float(), u.float()
         self.w_gate_up = torch.cat([g, u], dim=0).contiguous()
@@ -35,7 +42,7 @@ class GatedMLP(FeedForward):
         # tiles 0 .. I/16 - 1 of the tiled copy are gate rows, the rest up rows: what the fused SwiGLU kernel expects
         if self.intermediate_size % 16 == 0:
             self.w_gate_up, self.w_gate_up_tiled = ops.weight_forms(self.w_gate_up)
-        self.w_down, self.w_down_tiled = ops.weight_forms(weights.pop(prefix + ".down_proj.weight"))
+        self.w_down, self.w_down_tiled = ops.weight_forms(weights.pop(down))
 
     def capturable(self, batch):
         return True
@@ -80,3 +87,48 @@ class DenseMLP(FeedForward):
 
     def forward(self, x, batch):
         return ops.linear_few(ops.linear_xielu(x, self.w_up, self.act, tiled=self.w_up_tiled), self.w_down, self.w_down_tiled)
+
+
+class MoEMLP(FeedForward):
+    """``experts`` gated feed-forwards of inner size ``expert_size`` of which every token uses ``top``: those with the
+    largest choice scores s + correction among the experts of the ``groups_kept`` best of ``groups`` equal groups of
+    neighbours (a group's score is the largest choice score in it).  Weights: the chosen s over their sum (+ 1e-20),
+    times ``scale``.  Tensors: ``router [experts, H]``, ``correction [experts]``, ``e<i>.gate``, ``e<i>.up``,
+    ``e<i>.down``."""
+
+    def __init__(self, hidden_size: int, expert_size: int, experts: int, top: int, groups: int = 1, groups_kept: int = 1,
+                 scale: float = 1.0, names=("router", "correction", "e%d.gate", "e%d.up", "e%d.down")):
+        if experts <= 0 or groups <= 0 or experts % groups or not 0 < groups_kept <= groups or not 0 < top <= groups_kept * (experts // groups):
+            raise ValueError("a choice of %d among %d of %d groups of %d experts cannot be made" % (top, groups_kept, groups, experts))
+        self.hidden_size, self.expert_size, self.experts, self.top = hidden_size, expert_size, experts, top
+        self.groups, self.groups_kept, self.scale, self.names = groups, groups_kept, float(scale), names
+        self.w_router = self.correction = self.w_gate_up = self.w_down = None
+
+    def weight_specs(self, prefix):
+        H, F, E = self.hidden_size, self.expert_size, self.experts
+        router, corr, gate, up, down = (prefix + "." + n for n in self.names)
+        specs = [WeightSpec(router, (E, H)), WeightSpec(corr, (E,), "bias")]
+        for e in range(E):
+            specs += [WeightSpec(gate % e, (F, H)), WeightSpec(up % e, (F, H)), WeightSpec(down % e, (H, F))]
+        return specs
+
+    def bind(self, prefix, weights):
+        router, corr, gate, up, down = (prefix + "." + n for n in self.names)
+        # the router and its correction are float32 whatever the run: its scores decide, they are not activations
+        self.w_router = weights.pop(router).float().contiguous()
+        self.correction = weights[corr].float().contiguous()
+        E = self.experts
+        mats = [weights.pop(n % e) for e in range(E) for n in (gate, up, down)]
+        if len({m.dtype for m in mats}) > 1:
+            mats = [m.float() for m in mats]
+        # every expert's [gate rows | up rows] and its down matrix, the experts one after the other
+        self.w_gate_up = torch.stack([torch.cat([mats[3 * e], mats[3 * e + 1]], dim=0) for e in range(E)]).contiguous()
+        self.w_down = torch.stack([mats[3 * e + 2] for e in range(E)]).contiguous()
+
+    def capturable(self, batch):
+        return True
+
+    def forward(self, x, batch):
+        z = ops.linear(x, self.w_router, torch.float32)
+        ids, weights = ops.moe_route(z, self.correction, self.top, self.groups, self.groups_kept, self.scale)
+        return ops.moe_experts(x, ids, weights, self.w_gate_up, self.w_down)

@@ -11,24 +11,33 @@ from .base import Norm
 
 
 class RMSNorm(Norm):
-    def __init__(self, size: int, eps: float, suffix: str = ".weight"):
+    def __init__(self, size: int, eps: float, suffix: str = ".weight", offset: float = 0.0):
         """``suffix``: what the weight's name has behind the part's prefix (some checkpoints name the vector by the
-        prefix alone)."""
+        prefix alone).  ``offset``: the stored vector is centred on zero and multiplies as ``offset + w`` (1.0 for norms
+        whose weights are stored around zero); the sum is formed once, in float32, when the weights are bound."""
         self.size = size
         self.eps = float(eps)
         self.suffix = suffix
+        self.offset = float(offset)
         self.weight = None
 
     def weight_specs(self, prefix):
-        return [WeightSpec(prefix + self.suffix, (self.size,), "norm")]
+        # (the role says how random weights are drawn: around one, or around zero where the offset supplies the one)
+        return [WeightSpec(prefix + self.suffix, (self.size,), "bias" if self.offset else "norm")]
 
     def bind(self, prefix, weights):
         self.weight = weights[prefix + self.suffix]
+        if self.offset:
+            self.weight = (self.weight.float() + self.offset).contiguous()
 
     def capturable(self, batch):
         return True
 
     def add_norm(self, resid, delta, out_dtype, rows=None):
+        """``delta``: None, one addend, or a pair of addends (the results of two sublayers that read the same norm)."""
+        if isinstance(delta, (tuple, list)):
+            first, second = delta
+            return ops.add_rms_norm(resid, first, self.weight, self.eps, out_dtype, rows, delta2=second)
         return ops.add_rms_norm(resid, delta, self.weight, self.eps, out_dtype, rows)
 
     def add_normed(self, base, y, out=None, copy_dtype=None, mix=None):

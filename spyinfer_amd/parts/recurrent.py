@@ -4,6 +4,17 @@
 recurrence itself is a scan over the tokens:  z = sigmoid(Wz h + bz), u = Wx h + bx, candidate c = u + 1/2 where
 u >= 0 and sigmoid(u) where u < 0;  S_t = (1 - z) S_(t-1) + z c per channel;  output Wo (S_t * silu(Wg h)).  The state
 starts at zero, is float32 and lives in the request's slot; everything behind the projections is float32.
+
+``MLSTM`` and ``ChannelDelta`` keep a matrix per head, S [key size, value size], written with k v^T and read with
+S^T q.  ``MLSTM``: exponential input gate and sigmoid forget gate in the log domain, both capped by
+cap tanh(. / cap), with a running maximum m (from 0) that keeps the exponentials in range:
+m = max(f + m', i); S = e^(f + m' - m) S + e^(i - m) k v^T, n likewise with k alone;
+o = S^T q / (max(|n . q|, e^-m) + 1e-6), q scaled by 1/sqrt(key size); each head's o over its root mean square, times a
+weight, times sigmoid(Wg x), then the output projection.  ``ChannelDelta``: the gated delta rule; q, k and v pass a
+short causal convolution per channel and silu, q and k become unit vectors (q also times 1/sqrt(key size));
+S = diag(g) S with a decay g = exp(-exp(A_h) softplus(W2 W1 x + bias)) per head and key channel; u = beta (v - S^T k),
+beta = sigmoid(Wb x); S += k u^T; o = S^T q; each head's o over its root mean square, times a weight shared by the
+heads, times sigmoid(G2 G1 x), then the output projection.  The convolutions' last inputs are state of the request too.
 """
 from __future__ import annotations
 
@@ -81,4 +92,134 @@ class MinGRU(Mixer):
         zxg = ops.linear_few(x, self.w_zxg, self.w_zxg_tiled)
         n, multi = batch.shared["scan_pieces"]
         y = ops.mingru(zxg, self.b_z, self.b_x, cache.state, batch.array("scan_pieces"), n, multi, batch.array("slot_ids"))
+        return ops.linear_few(y, self.w_o, self.w_o_tiled)
+
+
+class MLSTM(Mixer):
+    def __init__(self, hidden_size: int, heads: int, dim: int, vdim: int, gate_cap: float, norm_eps: float,
+                 names=("q", "k", "v", "g", "o", "norm", "i", "i.b", "f", "f.b")):
+        self.hidden_size, self.heads, self.dim, self.vdim = hidden_size, heads, dim, vdim
+        self.gate_cap, self.norm_eps, self.names = float(gate_cap), float(norm_eps), names
+        if not self.gate_cap > 0.0:
+            raise ValueError("the gates' cap must be positive")
+        self.w_in = self.w_in_tiled = self.w_gates = self.w_o = self.w_o_tiled = self.b_i = self.b_f = self.norm = None
+
+    def weight_specs(self, prefix):
+        W, H, d, dv = self.hidden_size, self.heads, self.dim, self.vdim
+        q, k, v, g, o, norm, i, ib, f, fb = (prefix + "." + n for n in self.names)
+        return [WeightSpec(q, (H * d, W)), WeightSpec(k, (H * d, W)), WeightSpec(v, (H * dv, W)), WeightSpec(g, (H * dv, W)),
+                WeightSpec(o, (W, H * dv)), WeightSpec(norm, (H * dv,), "norm"), WeightSpec(i, (H, W)), WeightSpec(ib, (H,), "bias"),
+                WeightSpec(f, (H, W)), WeightSpec(fb, (H,), "bias")]
+
+    def bind(self, prefix, weights):
+        q, k, v, g, o, norm, i, ib, f, fb = (prefix + "." + n for n in self.names)
+        mats = [weights.pop(n) for n in (q, k, v, g)]
+        if len({m.dtype for m in mats}) > 1:
+            mats = [m.float() for m in mats]
+        # one product for the four wide projections: rows [q | k | v | g]; the two gates' products, which enter the
+        # recurrence's exponentials, come from a second, small product whose result stays float32
+        self.w_in, self.w_in_tiled = ops.weight_forms(torch.cat(mats, dim=0).contiguous())
+        del mats
+        gi, gf = weights.pop(i), weights.pop(f)
+        if gi.dtype != gf.dtype:
+            gi, gf = gi.float(), gf.float()
+        self.w_gates = torch.cat([gi, gf], dim=0).contiguous()
+        self.w_o, self.w_o_tiled = ops.weight_forms(weights.pop(o))
+        small = [weights[ib], weights[fb], weights[norm]]
+        if len({t.dtype for t in small}) > 1:
+            small = [t.float() for t in small]
+        self.b_i, self.b_f, self.norm = small
+
+    def cache_spec(self):
+        H, d, dv = self.heads, self.dim, self.vdim
+        return FixedState((H * (d * dv + d + 1),), "float32")
+
+    def capturable(self, batch):
+        return True
+
+    def forward(self, x, batch, cache, store=True):
+        if not store:
+            raise ValueError("a recurrence cannot run on another layer's state without writing it")
+        H, d, dv = self.heads, self.dim, self.vdim
+        proj = ops.linear_few(x, self.w_in, self.w_in_tiled)
+        gates = ops.linear(x, self.w_gates, torch.float32)
+        y = ops.mlstm(proj, 0, H * d, 2 * H * d, 2 * H * d + H * dv, gates, self.b_i, self.b_f, self.gate_cap, self.norm, self.norm_eps,
+                      cache.state, batch.array("cu_q"), batch.array("slot_ids"), H, d, dv)
+        return ops.linear_few(y, self.w_o, self.w_o_tiled)
+
+
+class ChannelDelta(Mixer):
+    def __init__(self, hidden_size: int, heads: int, kv_heads: int, dim: int, vdim: int, conv: int, norm_eps: float,
+                 decay_rank: int = None, gate_rank: int = None,
+                 names=("q", "k", "v", "b", "a1", "g1", "a2", "g2", "o", "q.conv", "k.conv", "v.conv", "A_log", "dt_bias", "norm")):
+        """``decay_rank``, ``gate_rank``: inner sizes of the two low-rank projections; None: whatever the stored
+        tensors have (a model folder is then needed: random weights cannot be drawn for an unknown size)."""
+        if heads % kv_heads:
+            raise ValueError("heads must be a multiple of kv_heads")
+        self.hidden_size, self.heads, self.kv_heads, self.dim, self.vdim, self.conv = hidden_size, heads, kv_heads, dim, vdim, conv
+        self.norm_eps, self.names = float(norm_eps), names
+        self.rank_a, self.rank_g = (-1 if decay_rank is None else decay_rank), (-1 if gate_rank is None else gate_rank)
+        if not 1 <= conv <= 8:
+            raise ValueError("the short convolution has 1 to 8 taps")
+        self.w_in = self.w_in_tiled = self.w_small = self.w_a2 = self.w_g2 = self.w_g2_tiled = self.w_o = self.w_o_tiled = None
+        self.taps = self.a_log = self.dt_bias = self.norm = None
+
+    def _channels(self):
+        return 2 * self.kv_heads * self.dim + self.heads * self.vdim
+
+    def weight_specs(self, prefix):
+        W, H, G, d, dv, n = self.hidden_size, self.heads, self.kv_heads, self.dim, self.vdim, self.conv
+        q, k, v, b, a1, g1, a2, g2, o, qc, kc, vc, alog, dtb, norm = (prefix + "." + x for x in self.names)
+        ra, rg = self.rank_a, self.rank_g
+        return [WeightSpec(q, (G * d, W)), WeightSpec(k, (G * d, W)), WeightSpec(v, (H * dv, W)), WeightSpec(b, (H, W)),
+                WeightSpec(a1, (ra, W)), WeightSpec(g1, (rg, W)), WeightSpec(a2, (H * d, ra)), WeightSpec(g2, (H * dv, rg)),
+                WeightSpec(o, (W, H * dv)), WeightSpec(qc, (G * d, n), "bias"), WeightSpec(kc, (G * d, n), "bias"),
+                WeightSpec(vc, (H * dv, n), "bias"), WeightSpec(alog, (H,), "bias"), WeightSpec(dtb, (H * d,), "bias"),
+                WeightSpec(norm, (dv,), "norm")]
+
+    def bind(self, prefix, weights):
+        q, k, v, b, a1, g1, a2, g2, o, qc, kc, vc, alog, dtb, norm = (prefix + "." + x for x in self.names)
+        mats = [weights.pop(n) for n in (q, k, v, g1)]
+        if len({m.dtype for m in mats}) > 1:
+            mats = [m.float() for m in mats]
+        if weights[a2].shape[1] != weights[a1].shape[0] or weights[g2].shape[1] != mats[3].shape[0]:
+            raise ValueError("%s: the inner sizes of the low-rank projections do not fit each other" % prefix)
+        # one product for the wide projections and the output gate's inner one: rows [q | k | v | g1]; what enters the
+        # recurrence's exponentials (beta, the decay's inner projection) comes from a second product that stays float32
+        self.w_in, self.w_in_tiled = ops.weight_forms(torch.cat(mats, dim=0).contiguous())
+        del mats
+        small = [weights.pop(b), weights.pop(a1)]
+        if small[0].dtype != small[1].dtype:
+            small = [t.float() for t in small]
+        self.w_small = torch.cat(small, dim=0).contiguous()
+        self.w_a2 = weights.pop(a2)
+        self.w_g2, self.w_g2_tiled = ops.weight_forms(weights.pop(g2))
+        self.w_o, self.w_o_tiled = ops.weight_forms(weights.pop(o))
+        taps = [weights[n] for n in (qc, kc, vc)]
+        vecs = [weights[alog], weights[dtb], weights[norm]]
+        if len({t.dtype for t in taps + vecs}) > 1:
+            taps, vecs = [t.float() for t in taps], [t.float() for t in vecs]
+        self.taps = torch.cat(taps, dim=0).contiguous()
+        self.a_log, self.dt_bias, self.norm = vecs
+
+    def cache_spec(self):
+        H, d, dv = self.heads, self.dim, self.vdim
+        return FixedState((H * d * dv + (self.conv - 1) * self._channels(),), "float32")
+
+    def capturable(self, batch):
+        return True
+
+    def forward(self, x, batch, cache, store=True):
+        if not store:
+            raise ValueError("a recurrence cannot run on another layer's state without writing it")
+        H, G, d, dv, C = self.heads, self.kv_heads, self.dim, self.vdim, self._channels()
+        proj = ops.linear_few(x, self.w_in, self.w_in_tiled)
+        small = ops.linear(x, self.w_small, torch.float32)                    # [beta | a1], float32
+        beta_pre = small[:, :H].contiguous()
+        dec_pre = ops.linear(small[:, H:].contiguous(), self.w_a2, torch.float32)
+        gate = ops.linear_few(proj[:, C:].contiguous(), self.w_g2, self.w_g2_tiled)
+        cu_q, slots = batch.array("cu_q"), batch.array("slot_ids")
+        qkv = ops.causal_conv_silu(proj[:, :C], self.taps, cache.state, H * d * dv, batch.array("token_entry"), cu_q, slots)
+        y = ops.delta_rule(qkv, beta_pre, dec_pre, self.a_log, self.dt_bias, gate, self.norm, self.norm_eps, cache.state, cu_q, slots,
+                           H, G, d, dv)
         return ops.linear_few(y, self.w_o, self.w_o_tiled)

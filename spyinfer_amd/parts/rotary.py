@@ -27,6 +27,10 @@ class RotaryEmbedding(PositionEncoding):
         if self.rotary_dim % 2 or not (0 < self.rotary_dim <= head_dim):
             raise ValueError("rotary_dim must be even and at most head_dim")
         self.scaling = dict(scaling) if scaling else None
+        #: a scaling with the keys {factor, low, high, original} goes by wavelength: a frequency whose wavelength is
+        #: shorter than original / high stays, one longer than original / low is divided by factor, and between the two
+        #: the divided and the plain frequency are blended linearly in original / wavelength (no factor on cos and sin)
+        self.by_wavelength = bool(self.scaling) and "low" in self.scaling and "high" in self.scaling
         self.cos = self.sin = None
         self._freq = None
 
@@ -38,6 +42,13 @@ class RotaryEmbedding(PositionEncoding):
         if self.scaling is None:
             return f, 1.0
         factor, original = float(self.scaling["factor"]), float(self.scaling["original"])
+        if self.by_wavelength:
+            low, high = float(self.scaling["low"]), float(self.scaling["high"])
+            wavelength = 2.0 * math.pi / f
+            blend = torch.clamp((original / wavelength - low) / (high - low), 0.0, 1.0) if high != low else (wavelength < original / high).double()
+            mixed = (1.0 - blend) * f / factor + blend * f
+            out = torch.where(wavelength < original / high, f, torch.where(wavelength > original / low, f / factor, mixed))
+            return out, 1.0
 
         def pair_of(turns: float) -> float:
             # the (fractional) pair index whose frequency makes ``turns`` turns in ``original`` positions

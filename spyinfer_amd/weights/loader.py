@@ -24,6 +24,7 @@ from .safetensors_io import open_folder
 @dataclasses.dataclass(frozen=True)
 class WeightSpec:
     name: str
+    #: an entry of -1 stands for a size that the stored tensor decides (an inner size that no configuration key names)
     shape: Tuple[int, ...]
     #: "matrix" (projection / embedding), "norm" (scale vector centred on 1), "bias" (vector centred on 0),
     #: "table" (integer table); the role decides how the random-weights mode draws the tensor
@@ -76,7 +77,7 @@ def load_weights(folder: str, specs: Iterable[WeightSpec], run_dtype: torch.dtyp
         if s.name not in where:
             continue
         dt, shape = where[s.name].info(s.name)
-        if tuple(shape) != tuple(s.shape):
+        if len(shape) != len(s.shape) or any(want >= 0 and want != got for want, got in zip(s.shape, shape)):
             wrong_shape.append((s.name, s.shape, shape))
         if s.role == "table":
             if dt.is_floating_point or dt == torch.bool:

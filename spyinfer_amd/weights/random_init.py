@@ -39,6 +39,8 @@ def random_tensors(specs: Iterable[WeightSpec], seed: int, dtype: torch.dtype = 
             continue
         if s.role not in ROLES:
             raise ValueError("tensor %s has the role %r; known roles: %s" % (s.name, s.role, ", ".join(ROLES)))
+        if any(n < 0 for n in s.shape):
+            raise ValueError("tensor %s has a size that only a stored tensor decides; random weights need it in the configuration" % s.name)
         g = _stream(seed, s.name)
         if s.role == "table":
             out[s.name] = torch.randint(0, table_range, s.shape, generator=g, dtype=torch.int32)

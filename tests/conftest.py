@@ -22,7 +22,8 @@ def emu_ops(monkeypatch):
     from tests.emu_ops import EmuOps
     emu = EmuOps()
     for name in ("embedding", "add_rms_norm", "rms_norm", "qk_norm_rope_store", "swiglu", "sample", "pair_embedding", "norm_residual",
-                 "depth_mix", "xielu", "mingru", "gemm_strided", "latent_prepare", "latent_attention"):
+                 "depth_mix", "xielu", "mingru", "gemm_strided", "latent_prepare", "latent_attention", "bias_rope_store", "sigmoid_gate",
+                 "mlstm", "causal_conv_silu", "delta_rule", "moe_route", "moe_experts"):
         monkeypatch.setattr(ops, name, getattr(emu, name))
 
     def linear(x, w, out_dtype=None, tiled=None, out=None):

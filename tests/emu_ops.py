@@ -8,10 +8,12 @@ import torch
 
 
 class EmuOps:
-    def embedding(self, ids, table):
-        return table[ids.long()].float()
+    def embedding(self, ids, table, scale=1.0):
+        return table[ids.long()].float() * scale
 
-    def add_rms_norm(self, resid, delta, weight, eps, out_dtype, rows=None):
+    def add_rms_norm(self, resid, delta, weight, eps, out_dtype, rows=None, delta2=None):
+        if delta is not None and delta2 is not None:
+            delta = delta.float() + delta2.float()
         if rows is None:
             if delta is not None:
                 resid += delta.float()
@@ -213,3 +215,128 @@ class EmuOps:
             pr = torch.softmax(sc, dim=1)[:, :len(keys)]
             out[t] = pr @ rows[:, :R]
         return out.to(out_dtype)
+
+    # ---- attention with biases, angles formed per call, an output gate ----
+    def bias_rope_store(self, x, n_q, n_kv, d, bias, freq, rotary_dim, positions, k_cache, v_cache, page_size, slots):
+        T = x.shape[0]
+        n = (n_q + 2 * n_kv) * d
+        f = x[:, :n].float()
+        if bias is not None:
+            f = f + bias.float()
+        q = f[:, :n_q * d].reshape(T, n_q, d)
+        k = f[:, n_q * d:(n_q + n_kv) * d].reshape(T, n_kv, d)
+        v = f[:, (n_q + n_kv) * d:].reshape(T, n_kv, d)
+        if rotary_dim:
+            q, k = self._rotate(q, positions, freq, 1.0, rotary_dim), self._rotate(k, positions, freq, 1.0, rotary_dim)
+        if slots is not None:
+            for t in range(T):
+                sl = int(slots[t])
+                if sl < 0:
+                    continue
+                k_cache[sl // page_size, :, sl % page_size, :] = k[t].to(k_cache.dtype)
+                v_cache[sl // page_size, :, :, sl % page_size] = v[t].to(v_cache.dtype)
+        return q.reshape(T, n_q * d).to(x.dtype)
+
+    def sigmoid_gate(self, y, gate):
+        y.copy_((y.float() * torch.sigmoid(gate.float())).to(y.dtype))
+        return y
+
+    # ---- matrix memories ----
+    def mlstm(self, x, q_off, k_off, v_off, g_off, gates, bi, bf, cap, norm_w, eps, state, cu_q, slot_ids, H, d, dv):
+        T = x.shape[0]
+        f = x.float()
+        out = torch.zeros((T, H, dv), dtype=torch.float32)
+        for s in range(slot_ids.shape[0]):
+            st = state[int(slot_ids[s])].view(H, d * dv + d + 1)
+            for h in range(H):
+                S, n, m = st[h, :d * dv].view(d, dv).clone(), st[h, d * dv:d * dv + d].clone(), float(st[h, -1])
+                for t in range(int(cu_q[s]), int(cu_q[s + 1])):
+                    q = f[t, q_off + h * d:q_off + (h + 1) * d] * d ** -0.5
+                    k = f[t, k_off + h * d:k_off + (h + 1) * d]
+                    v = f[t, v_off + h * dv:v_off + (h + 1) * dv]
+                    ig = cap * torch.tanh((gates[t, h] + bi[h].float()) / cap)
+                    fg = torch.nn.functional.logsigmoid(cap * torch.tanh((gates[t, H + h] + bf[h].float()) / cap))
+                    m_new = max(float(fg) + m, float(ig))
+                    a, b = torch.exp(fg + m - m_new), torch.exp(ig - m_new)
+                    S = a * S + b * torch.outer(k, v)
+                    n = a * n + b * k
+                    m = m_new
+                    den = max(abs(float(n @ q)), float(torch.exp(torch.tensor(-m)))) + 1e-6
+                    out[t, h] = (S.T @ q) / den
+                st[h, :d * dv] = S.reshape(-1)
+                st[h, d * dv:d * dv + d] = n
+                st[h, -1] = m
+        out = out * torch.rsqrt((out * out).mean(-1, keepdim=True) + eps)
+        g = f[:, g_off:g_off + H * dv]
+        return (out.reshape(T, H * dv) * norm_w.float() * torch.sigmoid(g)).to(x.dtype)
+
+    def causal_conv_silu(self, x, taps, state, keep_off, token_entry, cu_q, slot_ids):
+        T, C = x.shape
+        n = taps.shape[1]
+        f = x.float()
+        y = torch.zeros((T, C), dtype=torch.float32)
+        for s in range(slot_ids.shape[0]):
+            keep = state[int(slot_ids[s]), keep_off:keep_off + (n - 1) * C].view(n - 1, C)
+            t0, t1 = int(cu_q[s]), int(cu_q[s + 1])
+            rows = torch.cat([keep.clone(), f[t0:t1]], dim=0)
+            for t in range(t1 - t0):
+                acc = (rows[t:t + n] * taps.float().T).sum(0)
+                y[t0 + t] = acc * torch.sigmoid(acc)
+            if n > 1:
+                keep.copy_(rows[rows.shape[0] - (n - 1):])
+        return y.to(x.dtype)
+
+    def delta_rule(self, qkv, beta_pre, dec_pre, a_log, dt_bias, gate, norm_w, eps, state, cu_q, slot_ids, H, G, d, dv):
+        T = qkv.shape[0]
+        f = qkv.float()
+        q = f[:, :G * d].reshape(T, G, d)
+        k = f[:, G * d:2 * G * d].reshape(T, G, d)
+        v = f[:, 2 * G * d:].reshape(T, H, dv)
+        q = q / torch.sqrt((q * q).sum(-1, keepdim=True) + 1e-6) * d ** -0.5
+        k = k / torch.sqrt((k * k).sum(-1, keepdim=True) + 1e-6)
+        beta = torch.sigmoid(beta_pre)
+        dec = torch.exp(-torch.exp(a_log.float())[None, :, None] * torch.nn.functional.softplus(dec_pre + dt_bias.float()).view(T, H, d))
+        out = torch.zeros((T, H, dv), dtype=torch.float32)
+        for s in range(slot_ids.shape[0]):
+            st = state[int(slot_ids[s]), :H * d * dv].view(H, d, dv)
+            for h in range(H):
+                g = h // (H // G)
+                S = st[h].clone()
+                for t in range(int(cu_q[s]), int(cu_q[s + 1])):
+                    S = dec[t, h][:, None] * S
+                    u = beta[t, h] * (v[t, h] - S.T @ k[t, g])
+                    S = S + torch.outer(k[t, g], u)
+                    out[t, h] = S.T @ q[t, g]
+                st[h] = S
+        out = out * torch.rsqrt((out * out).mean(-1, keepdim=True) + eps) * norm_w.float()
+        return (out.reshape(T, H * dv) * torch.sigmoid(gate.float())).to(qkv.dtype)
+
+    # ---- mixture of experts ----
+    def moe_route(self, z, correction, top, groups, keep, scale):
+        T, E = z.shape
+        per = E // groups
+        ids = torch.zeros((T, top), dtype=torch.int32)
+        w = torch.zeros((T, top), dtype=torch.float32)
+        for t in range(T):
+            s = torch.softmax(z[t].float(), dim=0)
+            ch = (s + correction.float()).tolist()
+            best = sorted(range(groups), key=lambda g: (-max(ch[g * per:(g + 1) * per]), g))[:keep]
+            allowed = [e for e in range(E) if e // per in best]
+            chosen = sorted(allowed, key=lambda e: (-ch[e], e))[:top]
+            tot = sum(float(s[e]) for e in chosen) + 1e-20
+            for j, e in enumerate(chosen):
+                ids[t, j], w[t, j] = e, float(s[e]) / tot * scale
+        return ids, w
+
+    def moe_experts(self, x, ids, weights, w_gate_up, w_down):
+        T, K = x.shape
+        F = w_gate_up.shape[1] // 2
+        out = torch.zeros((T, K), dtype=torch.float32)
+        xf = x.float()
+        for t in range(T):
+            for j in range(ids.shape[1]):
+                e = int(ids[t, j])
+                gu = w_gate_up[e].float() @ xf[t]
+                act = (gu[:F] * torch.sigmoid(gu[:F]) * gu[F:]).to(x.dtype).float()
+                out[t] += weights[t, j] * (w_down[e].float() @ act)
+        return out.to(x.dtype)
