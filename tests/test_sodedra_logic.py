@@ -1,0 +1,144 @@
+"""Sodedra through the engine's own step function, cache manager, scheduler and entry point, with the CPU stand-in
+for the kernels: what is tested here is the logic around them (which pages and slots, which state, which kept
+inputs of the convolutions, which addends meet the stream), against the plain implementation."""
+import copy
+
+import pytest
+import torch
+
+from tests import replay_cases as rc
+from tests import sodedra_cases as sc
+from tests.plain.sodedra_plain import PlainSodedra
+
+CPU = ["--device", "cpu"]
+TOL = dict(atol=3e-4, rtol=3e-4)
+
+
+@pytest.fixture(scope="module")
+def folders(tmp_path_factory):
+    return {name: sc.write_model(str(tmp_path_factory.mktemp("sod_" + name)), cfg, seed, tweak, torch.float32)
+            for name, cfg, seed, tweak in (("a", sc.SOD_A, 3, None), ("b", sc.SOD_B, 4, None), ("a_sharp", sc.SOD_A, 5, sc.sharpen()),
+                                        ("a_memory", sc.SOD_A, 9, sc.long_memory()), ("a_router", sc.SOD_A, 11, sc.biased_router()))}
+
+
+def test_configuration_is_read_by_name_and_checked():
+    from spyinfer_amd.config import ConfigError, SodedraConfig
+    from spyinfer_amd.config.registry import architecture_of
+    assert architecture_of(sc.SOD_A).name == "Sodedra"
+    cfg = SodedraConfig.from_dict(copy.deepcopy(sc.SOD_A))
+    assert (cfg.vocab, cfg.width, cfg.embedding_scale, len(cfg.layers)) == (97, 48, 0.7, 7)
+    assert cfg.layers[0]["mixer"]["window"] == 9 and cfg.layers[3]["mixer"]["window"] is None and cfg.layers[2]["mlp"] is None
+    assert cfg.layers[3]["mixer"]["rot"]["scaling"] is None and cfg.layers[6]["mixer"]["rot"] is None
+    assert cfg.layers[0]["mlp"] == dict(kind="moe", ff=24, experts=8, top=3, groups=4, keep=2, scale=1.3)
+    for path, value in ((("layers", 0, "mixer", "kv_heads"), 3), (("layers", 0, "type"), "conv"), (("layers", 0, "mixer", "rot", "dims"), 3),
+                        (("layers", 0, "mixer", "rot", "dims"), 10), (("width",), None), (("layers", 1, "mlp", "kind"), "gated"),
+                        (("layers", 0, "mlp", "router", "top"), 5), (("layers", 0, "mlp", "router", "groups", "count"), 3),
+                        (("layers", 1, "mixer", "gate_cap"), 0.0), (("layers", 2, "mixer", "conv"), 9), (("norm", "eps"), 0.0)):
+        bad = copy.deepcopy(sc.SOD_A)
+        node = bad
+        for key in path[:-1]:
+            node = node[key]
+        node[path[-1]] = value
+        with pytest.raises(ConfigError):
+            SodedraConfig.from_dict(bad)
+
+
+def test_cache_kinds_follow_the_layers():
+    from spyinfer_amd.cache.spec import FixedState, PagedKV
+    from spyinfer_amd.config import SodedraConfig
+    from spyinfer_amd.models.sodedra import build_sodedra
+    model = build_sodedra(SodedraConfig.from_dict(copy.deepcopy(sc.SOD_A)))
+    specs = model.cache_specs()
+    # key and value heads of different sizes share one padded head size; windows give pages back, recurrences keep slots
+    assert specs[0] == PagedKV(2, 16, 9) and specs[3] == PagedKV(1, 16, None) and specs[6] == PagedKV(3, 4, 5)
+    assert specs[1] == FixedState((3 * (5 * 7 + 5 + 1),), "float32")
+    assert specs[2] == FixedState((4 * 6 * 5 + 2 * (2 * 2 * 6 + 4 * 5),), "float32")
+    assert model.lm_head.tied_to is model.embed
+
+
+def test_inner_sizes_that_no_key_names_come_from_the_tensors(folders, emu_ops, tmp_path):
+    """The delta rule's low-rank projections: without the optional keys the stored tensors decide."""
+    import json
+    import os
+    import shutil
+    folder = str(tmp_path / "m")
+    shutil.copytree(folders["a"], folder)
+    with open(os.path.join(folder, "config.json")) as f:
+        cfg = json.load(f)
+    for layer in cfg["layers"]:
+        layer["mixer"].pop("decay_rank", None)
+        layer["mixer"].pop("gate_rank", None)
+    with open(os.path.join(folder, "config.json"), "w") as f:
+        json.dump(cfg, f)
+    requests = rc.random_requests(97, [19], 3)
+    steps = rc.whole(requests)
+    rc.run_replay_inprocess(folder, "float32", str(tmp_path / "out"), steps, rc.max_live_tokens(steps), CPU)
+    rc.compare(rc.collect(str(tmp_path / "out"), steps, 97), sc.plain_logits(folders["a"], requests), what="ranks from tensors", **TOL)
+
+
+@pytest.mark.parametrize("name", ["a", "b", "a_sharp", "a_memory", "a_router"])
+@pytest.mark.parametrize("mode", ["whole", "bulk_tail", "portions", "mixed"])
+def test_schedules_equal_the_plain_implementation(folders, name, mode, tmp_path, emu_ops):
+    folder = folders[name]
+    requests = rc.random_requests(sc.vocab_of(folder), [41, 1, 2, 67, 23, 30, 52, 38, 45], 7)
+    steps = {"whole": rc.whole, "bulk_tail": lambda r: rc.bulk_tail(r, 12), "portions": rc.portions, "mixed": rc.mixed}[mode](requests)
+    if mode == "mixed":
+        rc.assert_mixed(steps, name)
+    rc.run_replay_inprocess(folder, "float32", str(tmp_path), steps, rc.max_live_tokens(steps), CPU + ["--kvcache-block-size", "8"])
+    rc.compare(rc.collect(str(tmp_path), steps, sc.vocab_of(folder)), sc.plain_logits(folder, requests), what="%s/%s" % (name, mode), **TOL)
+
+
+def test_pages_of_passed_windows_and_slots_go_back_and_are_used_again(folders, emu_ops):
+    from spyinfer_amd.engine.batch import StepEntry
+    from spyinfer_amd.engine.runner import ModelRunner, load_model
+    folder = folders["a_memory"]
+    model = load_model(folder, "float32", "cpu")
+    runner = ModelRunner(model, "float32", "cpu", 4, 40, 2, max_num_batched_tokens=1 << 20)
+    plain = PlainSodedra.from_folder(folder)
+    m = runner.manager
+    windowed = next(g for g in m.page_groups if g.spec.window == 9)
+    for turn in range(3):                          # the same two slots and the same pages serve three pairs of requests
+        reqs = rc.random_requests(97, [57, 33], 20 + turn)
+        held = {rid: m.admit(rid) for rid in reqs}
+        got = {rid: [] for rid in reqs}
+        fed = {rid: 0 for rid in reqs}
+        while any(fed[r] < len(reqs[r]) for r in reqs):
+            entries = []
+            for rid, toks in reqs.items():
+                n = min(5 if rid == "r0" else 1, len(toks) - fed[rid])
+                if n:
+                    m.reserve(held[rid], n)
+                    entries.append((rid, StepEntry(held[rid], toks[fed[rid]:fed[rid] + n], list(range(n)))))
+                    fed[rid] += n
+            logits = runner.step([e for _, e in entries])
+            r = 0
+            for rid, e in entries:
+                got[rid].append(logits[r:r + len(e.tokens)].clone())
+                r += len(e.tokens)
+            m.check()
+            assert all(len(rcache.pages_held(windowed.index)) <= (9 + 5) // 4 + 2 for rcache in held.values())
+        for rid, toks in reqs.items():
+            torch.testing.assert_close(torch.cat(got[rid]), plain.forward(toks).float(), **TOL)
+            m.release(held[rid])
+        assert m.num_free_pages() == [g.pool.num_pages for g in m.page_groups] and m.slots.num_free == 2
+
+
+def test_greedy_generation_through_the_entry_point(folders, emu_ops):
+    from spyinfer_amd.engine.llm_engine import LLMEngine
+    from spyinfer_amd.sampling import SamplingParams
+    folder = folders["a"]
+    plain = PlainSodedra.from_folder(folder)
+    prompts = list(rc.random_requests(97, [5, 17, 2, 30, 9], 9).values())
+    want = [plain.greedy(p, 10) for p in prompts]
+    for opts in (dict(), dict(max_num_batched_tokens=12, prefill_chunk=7, max_num_seqs=2), dict(num_kvcache_blocks=None)):
+        kw = dict(dtype="float32", max_model_len=64, num_kvcache_blocks=24, max_num_seqs=4, kvcache_block_size=8, device="cpu")
+        kw.update(opts)
+        eng = LLMEngine(folder, **kw)
+        assert eng.generate(prompts, SamplingParams(max_new_tokens=10, ignore_eos=True)) == want
+        eng.runner.manager.check()
+    # a pool too small for all requests at once: the request admitted last is preempted, gives its slot and pages back
+    # and later runs again from its first token, with the recurrences' state and the convolutions' kept inputs starting anew
+    eng = LLMEngine(folder, dtype="float32", max_model_len=64, num_kvcache_blocks=9, max_num_seqs=4, kvcache_block_size=8, device="cpu")
+    assert eng.generate(prompts, SamplingParams(max_new_tokens=10, ignore_eos=True)) == want
+    assert eng.scheduler.num_preemptions > 0
+    eng.runner.manager.check()
