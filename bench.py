@@ -22,6 +22,7 @@ Other workloads, each again one JSON line:
     python bench.py --shape 14b --serve 64                 # Qwen3-14B shape: 64 requests at once until all have ended
     python bench.py --shape 32b --batch 64 --prompt-len 4096 --context 4608 --points "" --steps 32 --warmup 4   # long keys at the 32B shape
     python bench.py --design sefevik [--design-sizes 1024,2048,4096] [--layers 8]   # Sefevik beside Qwen3 at equal size
+    python bench.py --design sodedra [--design-sizes 1024,2048,4096] [--layers 8]   # Sodedra beside Qwen3 at equal size
 """
 import argparse
 import json
@@ -70,9 +71,38 @@ def sefevik_shape(width: int, layers: int, vocab: int, window: int = 1024) -> di
                 embedding=dict(bigram=dict(buckets=65521, mul_prev=37, mul_cur=11)), layers=out)
 
 
+def sodedra_shape(width: int, layers: int, vocab: int, window: int = 1024) -> dict:
+    """A Sodedra configuration with the layer sizes of a real model of that width: attention heads of 128 with 64 rotated
+    dims and a quarter as many kv heads; matrix memories with keys of 128 (mLSTM: values of 256, half as many heads); a
+    dense feed-forward of three times the width, or 32 experts of a quarter of that of which a token uses four (as many
+    active weights); of every four layers an mLSTM, an attention with experts, a delta rule and an attention."""
+    heads = max(1, width // 128)
+    rot = dict(base=500000.0, dims=64, scaling=dict(factor=8.0, low=1.0, high=4.0, original=8192))
+    att = dict(heads=heads, kv_heads=max(1, heads // 4), dim=128, vdim=128, scale=128 ** -0.5, mask=dict(size=window), rot=rot)
+    dense = dict(kind="dense", ff=3 * width)
+    moe = dict(kind="moe", expert=dict(ff=3 * width // 4), router=dict(experts=32, top=4, scale=1.5, groups=dict(count=4, keep=2)))
+    out = []
+    for i in range(layers):
+        kind = i % 4
+        if kind == 0:
+            out.append(dict(type="mlstm", mixer=dict(heads=max(1, heads // 2), dim=128, vdim=256, gate_cap=15.0), mlp=dense))
+        elif kind == 1:
+            out.append(dict(type="attention", mixer=dict(att), mlp=moe))
+        elif kind == 2:
+            out.append(dict(type="channel_delta", mixer=dict(heads=heads, kv_heads=max(1, heads // 2), dim=128, vdim=128, conv=4,
+                                                             decay_rank=128, gate_rank=128), mlp=dense))
+        else:
+            out.append(dict(type="attention", mixer=dict(att), mlp=dense))
+    return dict(architecture="Sodedra", vocab=vocab, width=width, norm=dict(eps=1e-6), embedding=dict(scale=1.0), layers=out)
+
+
+DESIGN_SHAPES = {"sefevik": ("Sefevik", sefevik_shape), "sodedra": ("Sodedra", sodedra_shape)}
+
+
 def design_compare(args) -> int:
-    """Prefill (one portion of --prefill-tokens) and decode (batch 8 and 32, prompts of --prompt-len) of Sefevik and of
+    """Prefill (one portion of --prefill-tokens) and decode (batch 8 and 32, prompts of --prompt-len) of the design and of
     Qwen3 at equal width, layers, heads and feed-forward size; ONE JSON line."""
+    design, (design_name, shape_of) = args.design, DESIGN_SHAPES[args.design]
     import torch
 
     from spyinfer_amd.config.registry import architecture_of
@@ -91,7 +121,7 @@ def design_compare(args) -> int:
     results = {}
     for width in [int(x) for x in args.design_sizes.split(",") if x.strip()]:
         heads = max(1, width // 128)
-        raws = {"sefevik": sefevik_shape(width, layers, vocab),
+        raws = {design: shape_of(width, layers, vocab),
                 "qwen3": dict(MODEL_8B, num_hidden_layers=layers, hidden_size=width, num_attention_heads=heads,
                               num_key_value_heads=max(1, heads // 4), intermediate_size=3 * width, vocab_size=vocab)}
         for name, raw in raws.items():
@@ -143,11 +173,11 @@ def design_compare(args) -> int:
             torch.cuda.empty_cache()
     first = results[next(iter(results))]
     print(json.dumps({
-        "metric": "prefill and decode tok/s of Sefevik beside Qwen3 at equal width, layers, heads and feed-forward size",
-        "value": first["sefevik"]["decode_b8"]["tokens_per_s"], "unit": "tokens/s", "n_gpus": 1, "steps": max(16, args.steps // 4), "warmup": 8,
-        "ms_per_step": first["sefevik"]["decode_b8"]["ms_per_step"], "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "metric": "prefill and decode tok/s of %s beside Qwen3 at equal width, layers, heads and feed-forward size" % design_name,
+        "value": first[design]["decode_b8"]["tokens_per_s"], "unit": "tokens/s", "n_gpus": 1, "steps": max(16, args.steps // 4), "warmup": 8,
+        "ms_per_step": first[design]["decode_b8"]["ms_per_step"], "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "bf16" if args.dtype == "bfloat16" else "fp32", "data": "synthetic (random weights, uniform-random token ids)",
-        "config": {"model": "Sefevik / Qwen3 layer shapes", "layers": layers, "vocab": vocab, "prompt_len": args.prompt_len,
+        "config": {"model": "%s / Qwen3 layer shapes" % design_name, "layers": layers, "vocab": vocab, "prompt_len": args.prompt_len,
                    "prefill_tokens": args.prefill_tokens, "window": 1024, "graphs": not args.enforce_eager, "parallelism": "single GPU"},
         "widths": results}))
     return 0
@@ -179,7 +209,7 @@ def main() -> int:
     ap.add_argument("--serve", type=int, default=0, metavar="N",
                     help="instead of the decode steps: N requests arriving at once, prompts of 128..2048 and outputs of 64..512 "
                          "tokens (uniform), run until all have ended; the value is generated tokens per second of the whole run")
-    ap.add_argument("--design", default="", choices=["", "sefevik"],
+    ap.add_argument("--design", default="", choices=["", "sefevik", "sodedra"],
                     help="instead of the decode steps: prefill and decode throughput of that design at a few layer sizes "
                          "beside the Qwen3 shape of equal width, layers, heads and feed-forward size (--design-sizes)")
     ap.add_argument("--design-sizes", default="1024,2048,4096", help="widths for --design")

@@ -213,9 +213,150 @@ __global__ __launch_bounds__(256) void moe_gemm_kernel(TC* __restrict__ C, const
     }
 }
 
+
+// The same product on the matrix cores, bfloat16 operands and float32 sums (v_mfma_f32_16x16x32_bf16).  A block of four
+// waves takes up to MT neighbouring row tiles (16 sorted rows each) that belong to one expert, and a group of columns:
+// every wave owns its columns' rows of W (gated: 16 gate rows and the 16 up rows of the same columns; else 32 rows) and
+// walks K, loading its W fragments once per step and using them for all the row tiles, whose rows of A are gathered
+// through the pairs' tokens.  Operands go from memory straight into MFMA operand registers: lane (r = lane % 16,
+// g = lane / 16) holds row r, values k + 8 g .. + 7; the result tile is C^T: lane (r, g) holds C[row r][column 4 g + i].
+// A block whose MT tiles belong to several experts takes their runs in turn.
+typedef __attribute__((__vector_size__(8 * sizeof(short)))) short moe_bf16x8_t;
+typedef __attribute__((__vector_size__(4 * sizeof(float)))) float moe_f32x4_t;
+
+template <int MT, bool GATED, typename TC>
+__global__ __launch_bounds__(256) void moe_gemm_mfma_kernel(TC* __restrict__ C, const bf16_t* __restrict__ A, const bf16_t* __restrict__ W,
+                                                            const int* __restrict__ tile_expert, const int* __restrict__ sorted_pair,
+                                                            int gather, int max_tiles, int N, int K, long long w_stride) {
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63;
+    const int r = lane & 15, g = lane >> 4;
+    constexpr int NT = 2;
+    const int n0 = (blockIdx.y * 4 + wave) * (GATED ? 16 : 32);
+    if (n0 >= N) return;
+    int t = blockIdx.x * MT;
+    const int t_end = min(t + MT, max_tiles);
+    const moe_bf16x8_t zero8 = {0, 0, 0, 0, 0, 0, 0, 0};
+    while (t < t_end) {
+        const int e = __builtin_amdgcn_readfirstlane(tile_expert[t]);
+        if (e < 0) break;
+        int run = 1;
+        while (t + run < t_end && __builtin_amdgcn_readfirstlane(tile_expert[t + run]) == e) ++run;
+        const bf16_t* xrow[MT];
+        bool xok[MT];
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt) {
+            xok[mt] = false;
+            xrow[mt] = A;
+            if (mt < run) {
+                const int row = (t + mt) * MOE_TM + r;
+                const int p = sorted_pair[row];
+                xok[mt] = p >= 0;
+                const int src = gather > 0 ? p / gather : row;
+                xrow[mt] = A + (size_t)(p >= 0 ? src : 0) * K + 8 * g;
+            }
+        }
+        const bf16_t* We = W + (size_t)e * w_stride;
+        const bf16_t* wrow[NT];
+#pragma unroll
+        for (int nt = 0; nt < NT; ++nt) {
+            const int row = GATED ? nt * N + min(n0 + r, N - 1) : min(n0 + nt * 16 + r, N - 1);
+            wrow[nt] = We + (size_t)row * K + 8 * g;
+        }
+        moe_f32x4_t acc[NT][MT];
+#pragma unroll
+        for (int nt = 0; nt < NT; ++nt)
+#pragma unroll
+            for (int mt = 0; mt < MT; ++mt) acc[nt][mt] = moe_f32x4_t{0.f, 0.f, 0.f, 0.f};
+        int k = 0;
+        for (; k + 128 <= K; k += 128) {
+            moe_bf16x8_t a[NT][4], b[MT][4];
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+#pragma unroll
+                for (int nt = 0; nt < NT; ++nt) a[nt][j] = *reinterpret_cast<const moe_bf16x8_t*>(wrow[nt] + k + 32 * j);
+#pragma unroll
+                for (int mt = 0; mt < MT; ++mt) b[mt][j] = xok[mt] ? *reinterpret_cast<const moe_bf16x8_t*>(xrow[mt] + k + 32 * j) : zero8;
+            }
+#pragma unroll
+            for (int j = 0; j < 4; ++j)
+#pragma unroll
+                for (int mt = 0; mt < MT; ++mt)
+                    if (mt < run) {
+#pragma unroll
+                        for (int nt = 0; nt < NT; ++nt) acc[nt][mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[nt][j], b[mt][j], acc[nt][mt], 0, 0, 0);
+                    }
+        }
+        for (; k < K; k += 32) {                  // the rest of K (a multiple of 8)
+            const bool kok = k + 8 * g < K;
+            moe_bf16x8_t a[NT], b[MT];
+#pragma unroll
+            for (int nt = 0; nt < NT; ++nt) a[nt] = kok ? *reinterpret_cast<const moe_bf16x8_t*>(wrow[nt] + k) : zero8;
+#pragma unroll
+            for (int mt = 0; mt < MT; ++mt) b[mt] = (kok && xok[mt]) ? *reinterpret_cast<const moe_bf16x8_t*>(xrow[mt] + k) : zero8;
+#pragma unroll
+            for (int mt = 0; mt < MT; ++mt)
+                if (mt < run) {
+#pragma unroll
+                    for (int nt = 0; nt < NT; ++nt) acc[nt][mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[nt], b[mt], acc[nt][mt], 0, 0, 0);
+                }
+        }
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt) {
+            if (mt >= run || !xok[mt]) continue;
+            const size_t row = (size_t)(t + mt) * MOE_TM + r;
+            if (GATED) {
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    const int col = n0 + 4 * g + i;
+                    if (col < N) {
+                        const float gt = acc[0][mt][i];
+                        C[row * N + col] = from_f32<TC>(gt / (1.0f + expf(-gt)) * acc[1][mt][i]);
+                    }
+                }
+            } else {
+#pragma unroll
+                for (int nt = 0; nt < NT; ++nt)
+#pragma unroll
+                    for (int i = 0; i < 4; ++i) {
+                        const int col = n0 + nt * 16 + 4 * g + i;
+                        if (col < N) C[row * N + col] = from_f32<TC>(acc[nt][mt][i]);
+                    }
+            }
+        }
+        t += run;
+    }
+}
+
+template <int MT>
+static int moe_gemm_mfma_launch(void* C, int c_dtype, const void* A, const void* W, const int* tile_expert, const int* sorted_pair,
+                                int gather, int gated, int max_tiles, int N, int K, hipStream_t st) {
+    const long long ws = (long long)(gated ? 2 : 1) * N * K;
+    const int cols = gated ? 64 : 128;
+    const dim3 grid((max_tiles + MT - 1) / MT, (N + cols - 1) / cols);
+    SPY_REQUIRE(grid.y <= 65535, "spy_moe_gemm: too many columns");
+    if (gated) {
+        SPY_DISPATCH(c_dtype, TC, (moe_gemm_mfma_kernel<MT, true, TC><<<grid, 256, 0, st>>>((TC*)C, (const bf16_t*)A, (const bf16_t*)W, tile_expert,
+                                                                                           sorted_pair, gather, max_tiles, N, K, ws)));
+    } else {
+        SPY_DISPATCH(c_dtype, TC, (moe_gemm_mfma_kernel<MT, false, TC><<<grid, 256, 0, st>>>((TC*)C, (const bf16_t*)A, (const bf16_t*)W, tile_expert,
+                                                                                            sorted_pair, gather, max_tiles, N, K, ws)));
+    }
+    return 0;
+}
+
 extern "C" int spy_moe_gemm(void* C, int c_dtype, const void* A, int a_dtype, const void* W, int w_dtype, const int* tile_expert,
-                            const int* sorted_pair, int gather, int gated, int max_tiles, int E, int N, int K, hipStream_t st) {
-    SPY_REQUIRE(max_tiles > 0 && max_tiles <= 65535 && E > 0 && N > 0 && K > 0 && gather >= 0, "spy_moe_gemm: bad sizes (%d tiles)", max_tiles);
+                            const int* sorted_pair, int gather, int gated, int max_tiles, int E, int N, int K, int tiles_per_block,
+                            hipStream_t st) {
+    SPY_REQUIRE(max_tiles > 0 && E > 0 && N > 0 && K > 0 && gather >= 0, "spy_moe_gemm: bad sizes (%d tiles)", max_tiles);
+    // bfloat16 operands in 16-byte pieces: the matrix cores; tiles_per_block: 0 = the plain float32 kernel
+    if (tiles_per_block > 0 && a_dtype == SPY_BF16 && w_dtype == SPY_BF16 && K % 8 == 0 && ((uintptr_t)A % 16) == 0 && ((uintptr_t)W % 16) == 0) {
+        const int rc = tiles_per_block >= 8 ? moe_gemm_mfma_launch<8>(C, c_dtype, A, W, tile_expert, sorted_pair, gather, gated, max_tiles, N, K, st)
+                                            : moe_gemm_mfma_launch<1>(C, c_dtype, A, W, tile_expert, sorted_pair, gather, gated, max_tiles, N, K, st);
+        if (rc) return rc;
+        SPY_CHECK_LAUNCH("spy_moe_gemm (mfma)");
+        return 0;
+    }
+    SPY_REQUIRE(max_tiles <= 65535, "spy_moe_gemm: %d tiles are too many for the plain kernel", max_tiles);
     const dim3 grid((N + MG_TN - 1) / MG_TN, max_tiles);
     const long long ws = (long long)(gated ? 2 : 1) * N * K;
     if (gated) {

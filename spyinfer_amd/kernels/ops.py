@@ -1304,6 +1304,9 @@ def moe_route(z: torch.Tensor, correction: torch.Tensor, top: int, groups: int, 
     return ids, w
 
 
+MOE_MFMA = True            # False forces the plain float32 kernel for bfloat16 too (tests flip it; nothing else does)
+
+
 def moe_experts(x: torch.Tensor, ids: torch.Tensor, weights: torch.Tensor, w_gate_up: torch.Tensor, w_down: torch.Tensor) -> torch.Tensor:
     """out[t] = sum_k weights[t, k] * down_e( silu(gate_e x[t]) * up_e x[t] ), e = ids[t, k]; ``w_gate_up [E, 2 F, K]`` =
     every expert's [gate rows | up rows], ``w_down [E, K, F]``.  The (token, choice) pairs are sorted by expert on the
@@ -1329,14 +1332,17 @@ def moe_experts(x: torch.Tensor, ids: torch.Tensor, weights: torch.Tensor, w_gat
     tile_expert = torch.empty((max_tiles,), dtype=torch.int32, device=dev)
     hip().call("spy_moe_align", _ptr(sorted_pair), _ptr(pair_row), _ptr(tile_expert), _ptr(ids), ctypes.c_int(P), ctypes.c_int(E),
                ctypes.c_int(max_tiles), _Hip.stream())
+    # bfloat16: the matrix cores, a block taking one row tile of an expert when the experts have few rows (decoding:
+    # blocks for the whole device), up to eight when they have many (an expert's matrices are read once per 128 rows)
+    per_block = 0 if not MOE_MFMA or x.dtype != torch.bfloat16 or w_gate_up.dtype != torch.bfloat16 else (8 if P >= 16 * E else 1)
     act = torch.empty((max_tiles * tm, F), dtype=x.dtype, device=dev)
     hip().call("spy_moe_gemm", _ptr(act), _code(act, "act"), _ptr(x), _code(x, "x"), _ptr(w_gate_up), _code(w_gate_up, "expert matrices"),
                _ptr(tile_expert), _ptr(sorted_pair), ctypes.c_int(top), ctypes.c_int(1), ctypes.c_int(max_tiles), ctypes.c_int(E), ctypes.c_int(F),
-               ctypes.c_int(K), _Hip.stream())
+               ctypes.c_int(K), ctypes.c_int(per_block), _Hip.stream())
     y = torch.empty((max_tiles * tm, K), dtype=torch.float32, device=dev)
     hip().call("spy_moe_gemm", _ptr(y), F32, _ptr(act), _code(act, "act"), _ptr(w_down), _code(w_down, "expert matrices"), _ptr(tile_expert),
                _ptr(sorted_pair), ctypes.c_int(0), ctypes.c_int(0), ctypes.c_int(max_tiles), ctypes.c_int(E), ctypes.c_int(K), ctypes.c_int(F),
-               _Hip.stream())
+               ctypes.c_int(per_block), _Hip.stream())
     hip().call("spy_moe_combine", _ptr(out), _code(out, "out"), _ptr(y), _ptr(weights), _ptr(pair_row), ctypes.c_int(T), ctypes.c_int(top),
                ctypes.c_int(K), _Hip.stream())
     return out

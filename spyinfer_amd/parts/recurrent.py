@@ -120,10 +120,8 @@ class MLSTM(Mixer):
         # recurrence's exponentials, come from a second, small product whose result stays float32
         self.w_in, self.w_in_tiled = ops.weight_forms(torch.cat(mats, dim=0).contiguous())
         del mats
-        gi, gf = weights.pop(i), weights.pop(f)
-        if gi.dtype != gf.dtype:
-            gi, gf = gi.float(), gf.float()
-        self.w_gates = torch.cat([gi, gf], dim=0).contiguous()
+        # (kept float32: a product of a few rows of any shape, through the true 32-bit kernel in both runs)
+        self.w_gates = torch.cat([weights.pop(i).float(), weights.pop(f).float()], dim=0).contiguous()
         self.w_o, self.w_o_tiled = ops.weight_forms(weights.pop(o))
         small = [weights[ib], weights[fb], weights[norm]]
         if len({t.dtype for t in small}) > 1:
@@ -188,11 +186,8 @@ class ChannelDelta(Mixer):
         # recurrence's exponentials (beta, the decay's inner projection) comes from a second product that stays float32
         self.w_in, self.w_in_tiled = ops.weight_forms(torch.cat(mats, dim=0).contiguous())
         del mats
-        small = [weights.pop(b), weights.pop(a1)]
-        if small[0].dtype != small[1].dtype:
-            small = [t.float() for t in small]
-        self.w_small = torch.cat(small, dim=0).contiguous()
-        self.w_a2 = weights.pop(a2)
+        self.w_small = torch.cat([weights.pop(b).float(), weights.pop(a1).float()], dim=0).contiguous()
+        self.w_a2 = weights.pop(a2).float().contiguous()
         self.w_g2, self.w_g2_tiled = ops.weight_forms(weights.pop(g2))
         self.w_o, self.w_o_tiled = ops.weight_forms(weights.pop(o))
         taps = [weights[n] for n in (qc, kc, vc)]
