@@ -1,7 +1,9 @@
 // Recurrent mixers whose state is a matrix per head, S [d, dv] in float32 in the request's slot: a write k v^T per
-// token, a read-out S^T q.  One block per (entry, head); thread j owns column j of S (the d values that belong to value
-// channel j) in registers and walks the entry's tokens; the token's key and query go through LDS.  Everything behind
-// the projections is float32; the result is rounded once, at its store.
+// token, a read-out S^T q.  One wave per (entry, head, slice of 64 value channels); lane j owns one column of S (the d
+// values that belong to its value channel) in registers and walks the entry's tokens; the token's key and query go
+// through LDS, and the next token's operands are asked for before this token's arithmetic.  The read-outs leave as
+// float32; a second kernel norms every head over all its slices, applies weight and gate and rounds once.
+// Everything behind the projections is float32.
 //
 //   mlstm:       S = a S + b k v^T, n = a n + b k with a = exp(f + m' - m), b = exp(i - m), m = max(f + m', i) (m starts at
 //                0), i and f capped log gates; o = S^T q / (max(|n . q|, exp(-m)) + 1e-6); then o / rms(o) * w * sigmoid(g).
@@ -14,116 +16,151 @@
 __device__ __forceinline__ float mm_sigmoid(float x) { return 1.0f / (1.0f + expf(-x)); }
 __device__ __forceinline__ float mm_logsigmoid(float x) { return fminf(x, 0.f) - log1pf(expf(-fabsf(x))); }
 
-// sums of two values over the block; red holds 2 * 16 floats
-__device__ __forceinline__ void block_sum2(float& a, float& b, float* red) {
-    a = wave_sum(a);
-    b = wave_sum(b);
-    const int lane = threadIdx.x & 63, w = threadIdx.x >> 6, nw = (blockDim.x + 63) >> 6;
-    if (lane == 0) { red[w] = a; red[16 + w] = b; }
-    __syncthreads();
-    float x = 0.f, y = 0.f;
-    for (int i = 0; i < nw; ++i) { x += red[i]; y += red[16 + i]; }
-    a = x;
-    b = y;
+#define MM_SLICE 64
+
+// out[t, h, j] = o[t, h, j] / sqrt(mean_j(o[t, h, :]^2) + eps) * w[(per_head ? h dv : 0) + j] * sigmoid(gate[t, h dv + j]);
+// one block per (token, head)
+template <typename TA, typename TW>
+__global__ void head_norm_gate_kernel(TA* __restrict__ out, const float* __restrict__ o, const TA* __restrict__ gate, long long gs,
+                                      const TW* __restrict__ w, int per_head, float eps, int H, int dv) {
+    __shared__ float red[16];
+    const int t = blockIdx.x, h = blockIdx.y;
+    const float* row = o + ((size_t)t * H + h) * dv;
+    float ss = 0.f;
+    for (int j = threadIdx.x; j < dv; j += blockDim.x) ss += row[j] * row[j];
+    ss = block_sum(ss, red);
+    const float r = 1.0f / sqrtf(ss / (float)dv + eps);
+    const TA* g = gate + (size_t)t * gs + (size_t)h * dv;
+    const TW* wr = w + (per_head ? (size_t)h * dv : 0);
+    TA* dst = out + ((size_t)t * H + h) * dv;
+    for (int j = threadIdx.x; j < dv; j += blockDim.x)
+        dst[j] = from_f32<TA>(((row[j] * r) * to_f32<TW>(wr[j])) * mm_sigmoid(to_f32<TA>(g[j])));
 }
 
 // ---- mLSTM ----------------------------------------------------------------------------------------------------------
 // x: rows of the fused projection, xs values apart; q at column q_off (H heads of d), k at k_off, v at v_off (H heads of
-// dv), the output gate's rows at g_off (H dv).  gates [T, 2 H] float32: the raw products of the input and the forget
-// gate.  state [slots][H][d dv + d + 1]: S (row dd, column j at dd dv + j), n, m.
-template <typename TA, typename TW, int DR, int BT>
-__global__ __launch_bounds__(BT) void mlstm_kernel(
-    TA* __restrict__ out, float* __restrict__ state, const TA* __restrict__ x, long long xs, int q_off, int k_off, int v_off,
-    int g_off, const float* __restrict__ gates, const TW* __restrict__ bi, const TW* __restrict__ bf, float cap,
-    const TW* __restrict__ norm_w, float eps, const int* __restrict__ cu_q, const int* __restrict__ slot_ids, int num_slots, int H,
-    int d, int dv) {
-    __shared__ float ks[DR], qs[DR], red[32];
-    const int s = blockIdx.x, h = blockIdx.y, j = threadIdx.x;
+// dv).  gates [T, 2 H] float32: the raw products of the input and the forget gate.  state [slots][H][d dv + NS (d + 1)]:
+// S (row dd, column j at dd dv + j), then for every slice of 64 columns its own copy of n and m (the slices' waves do
+// not wait for each other, so none may read what another has already moved on).
+template <typename TA, typename TW, int DR>
+__global__ __launch_bounds__(MM_SLICE) void mlstm_kernel(
+    float* __restrict__ o_out, float* __restrict__ state, const TA* __restrict__ x, long long xs, int q_off, int k_off, int v_off,
+    const float* __restrict__ gates, const TW* __restrict__ bi, const TW* __restrict__ bf, float cap, const int* __restrict__ cu_q,
+    const int* __restrict__ slot_ids, int num_slots, int H, int d, int dv, int NS) {
+    __shared__ __align__(16) float ks[DR], qs[DR];
+    constexpr int R = DR / MM_SLICE;
+    const int s = blockIdx.x, h = blockIdx.y, c = blockIdx.z, lane = threadIdx.x;
+    const int j = c * MM_SLICE + lane;
     const int slot = slot_ids[s];
     if (slot < 0 || slot >= num_slots) return;
-    const size_t head_state = (size_t)d * dv + d + 1;
+    const size_t head_state = (size_t)d * dv + (size_t)NS * (d + 1);
     float* st = state + ((size_t)slot * H + h) * head_state;
+    float* nm = st + (size_t)d * dv + (size_t)c * (d + 1);
+    const bool col = j < dv;
     float S[DR];
-    const bool col = j < dv, row = j < d;
 #pragma unroll
     for (int dd = 0; dd < DR; ++dd) S[dd] = (col && dd < d) ? st[(size_t)dd * dv + j] : 0.f;
-    float n = row ? st[(size_t)d * dv + j] : 0.f;
-    float m = st[(size_t)d * dv + d];
+    float n[R];
+#pragma unroll
+    for (int i = 0; i < R; ++i) {
+        const int idx = lane + MM_SLICE * i;
+        n[i] = idx < d ? nm[idx] : 0.f;
+        ks[idx] = 0.f;
+        qs[idx] = 0.f;
+    }
+    float m = nm[d];
     const float b_i = to_f32<TW>(bi[h]), b_f = to_f32<TW>(bf[h]);
-    const float wn = col ? to_f32<TW>(norm_w[(size_t)h * dv + j]) : 0.f;
     const float qscale = 1.0f / sqrtf((float)d);
-    const int t1 = cu_q[s + 1];
-    for (int t = cu_q[s]; t < t1; ++t) {
-        const TA* xr = x + (size_t)t * xs;
-        if (row) {
-            ks[j] = to_f32<TA>(xr[k_off + (size_t)h * d + j]);
-            qs[j] = to_f32<TA>(xr[q_off + (size_t)h * d + j]) * qscale;
+    const int t0 = cu_q[s], t1 = cu_q[s + 1];
+    float kc[R], qc[R], vc = 0.f, gic = 0.f, gfc = 0.f;
+    float kn[R], qn[R], vn = 0.f, gin = 0.f, gfn = 0.f;
+#define MLSTM_LOAD(K, Q, V, GI, GF, TT)                                                        \
+    {                                                                                          \
+        const TA* xr_ = x + (size_t)(TT) * xs;                                                 \
+        _Pragma("unroll") for (int i = 0; i < R; ++i) {                                        \
+            const int idx = lane + MM_SLICE * i;                                               \
+            K[i] = idx < d ? to_f32<TA>(xr_[k_off + (size_t)h * d + idx]) : 0.f;               \
+            Q[i] = idx < d ? to_f32<TA>(xr_[q_off + (size_t)h * d + idx]) * qscale : 0.f;      \
+        }                                                                                      \
+        V = col ? to_f32<TA>(xr_[v_off + (size_t)h * dv + j]) : 0.f;                           \
+        GI = gates[(size_t)(TT) * 2 * H + h];                                                  \
+        GF = gates[(size_t)(TT) * 2 * H + H + h];                                              \
+    }
+    if (t0 < t1) MLSTM_LOAD(kc, qc, vc, gic, gfc, t0)
+    for (int t = t0; t < t1; ++t) {
+        if (t + 1 < t1) MLSTM_LOAD(kn, qn, vn, gin, gfn, t + 1)
+#pragma unroll
+        for (int i = 0; i < R; ++i) {
+            const int idx = lane + MM_SLICE * i;
+            if (idx < d) { ks[idx] = kc[i]; qs[idx] = qc[i]; }
         }
-        const float vj = col ? to_f32<TA>(xr[v_off + (size_t)h * dv + j]) : 0.f;
-        const float gj = col ? to_f32<TA>(xr[g_off + (size_t)h * dv + j]) : 0.f;
-        const float ig = cap * tanhf((gates[(size_t)t * 2 * H + h] + b_i) / cap);
-        const float fg = mm_logsigmoid(cap * tanhf((gates[(size_t)t * 2 * H + H + h] + b_f) / cap));
+        const float ig = cap * tanhf((gic + b_i) / cap);
+        const float fg = mm_logsigmoid(cap * tanhf((gfc + b_f) / cap));
         const float m_new = fmaxf(fg + m, ig);
         const float a = expf(fg + m - m_new), b = expf(ig - m_new);
         m = m_new;
         __syncthreads();
-        float acc = 0.f, nq = 0.f;
-        const float bv = b * vj;
+        float acc = 0.f;
+        const float bv = b * vc;
 #pragma unroll
-        for (int dd = 0; dd < DR; ++dd) {
+        for (int dd = 0; dd < DR; dd += 4) {
             if (dd < d) {
-                S[dd] = fmaf(a, S[dd], ks[dd] * bv);
-                acc = fmaf(S[dd], qs[dd], acc);
+                const float4 k4 = *reinterpret_cast<const float4*>(ks + dd), q4 = *reinterpret_cast<const float4*>(qs + dd);
+                S[dd] = fmaf(a, S[dd], k4.x * bv);         acc = fmaf(S[dd], q4.x, acc);
+                S[dd + 1] = fmaf(a, S[dd + 1], k4.y * bv); acc = fmaf(S[dd + 1], q4.y, acc);
+                S[dd + 2] = fmaf(a, S[dd + 2], k4.z * bv); acc = fmaf(S[dd + 2], q4.z, acc);
+                S[dd + 3] = fmaf(a, S[dd + 3], k4.w * bv); acc = fmaf(S[dd + 3], q4.w, acc);
             }
         }
-        if (row) {
-            n = fmaf(a, n, b * ks[j]);
-            nq = n * qs[j];
+        float nq = 0.f;
+#pragma unroll
+        for (int i = 0; i < R; ++i) {
+            n[i] = fmaf(a, n[i], b * kc[i]);
+            nq = fmaf(n[i], qc[i], nq);
         }
-        float ss = col ? acc * acc : 0.f;
-        block_sum2(nq, ss, red);
+        nq = wave_sum(nq);
         const float den = fmaxf(fabsf(nq), expf(-m)) + 1e-6f;
-        if (col) {
-            const float o = acc / den;
-            const float r = 1.0f / sqrtf(ss / (den * den) / (float)dv + eps);
-            out[(size_t)t * H * dv + (size_t)h * dv + j] = from_f32<TA>(((o * r) * wn) * mm_sigmoid(gj));
-        }
+        if (col) o_out[((size_t)t * H + h) * dv + j] = acc / den;
+        __syncthreads();
+#pragma unroll
+        for (int i = 0; i < R; ++i) { kc[i] = kn[i]; qc[i] = qn[i]; }
+        vc = vn; gic = gin; gfc = gfn;
     }
+#undef MLSTM_LOAD
 #pragma unroll
     for (int dd = 0; dd < DR; ++dd)
         if (col && dd < d) st[(size_t)dd * dv + j] = S[dd];
-    if (row) st[(size_t)d * dv + j] = n;
-    if (j == 0) st[(size_t)d * dv + d] = m;
+#pragma unroll
+    for (int i = 0; i < R; ++i) {
+        const int idx = lane + MM_SLICE * i;
+        if (idx < d) nm[idx] = n[i];
+    }
+    if (lane == 0) nm[d] = m;
 }
 
-#define MM_LAUNCH(KERNEL, ...)                                                                                  \
-    do {                                                                                                        \
-        const int need_ = d > dv ? d : dv;                                                                      \
-        const int bt_ = need_ <= 64 ? 64 : (need_ <= 256 ? 256 : 1024);                                        \
-        const int threads_ = (need_ + 63) / 64 * 64;                                                            \
-        if (d <= 64) {                                                                                          \
-            if (bt_ == 64) KERNEL<TA, TW, 64, 64><<<grid, threads_, 0, st>>>(__VA_ARGS__);                      \
-            else if (bt_ == 256) KERNEL<TA, TW, 64, 256><<<grid, threads_, 0, st>>>(__VA_ARGS__);               \
-            else KERNEL<TA, TW, 64, 1024><<<grid, threads_, 0, st>>>(__VA_ARGS__);                              \
-        } else if (d <= 128) {                                                                                  \
-            if (bt_ <= 256) KERNEL<TA, TW, 128, 256><<<grid, threads_, 0, st>>>(__VA_ARGS__);                   \
-            else KERNEL<TA, TW, 128, 1024><<<grid, threads_, 0, st>>>(__VA_ARGS__);                             \
-        } else {                                                                                                \
-            if (bt_ <= 256) KERNEL<TA, TW, 256, 256><<<grid, threads_, 0, st>>>(__VA_ARGS__);                   \
-            else KERNEL<TA, TW, 256, 1024><<<grid, threads_, 0, st>>>(__VA_ARGS__);                             \
-        }                                                                                                       \
+#define MM_LAUNCH(KERNEL, ...)                                                              \
+    do {                                                                                    \
+        if (d <= 64) KERNEL<TA, TW, 64><<<grid, MM_SLICE, 0, st>>>(__VA_ARGS__);            \
+        else if (d <= 128) KERNEL<TA, TW, 128><<<grid, MM_SLICE, 0, st>>>(__VA_ARGS__);     \
+        else KERNEL<TA, TW, 256><<<grid, MM_SLICE, 0, st>>>(__VA_ARGS__);                   \
     } while (0)
 
-extern "C" int spy_mlstm(void* out, float* state, const void* x, long long xs, int dtype, int q_off, int k_off, int v_off, int g_off,
-                         const float* gates, const void* bi, const void* bf, int w_dtype, float cap, const void* norm_w, float eps,
-                         const int* cu_q, const int* slot_ids, int num_slots, int S, int T, int H, int d, int dv, hipStream_t st) {
-    SPY_REQUIRE(S > 0 && T > 0 && H > 0 && d > 0 && dv > 0 && num_slots > 0, "spy_mlstm: empty operand");
+extern "C" int spy_mlstm(void* out, float* o_tmp, float* state, const void* x, long long xs, int dtype, int q_off, int k_off, int v_off,
+                         int g_off, const float* gates, const void* bi, const void* bf, int w_dtype, float cap, const void* norm_w,
+                         float eps, const int* cu_q, const int* slot_ids, int num_slots, int S, int T, int H, int d, int dv, hipStream_t st) {
+    SPY_REQUIRE(S > 0 && T > 0 && H > 0 && d > 0 && dv > 0 && num_slots > 0 && o_tmp, "spy_mlstm: empty operand");
     SPY_REQUIRE(d <= 256 && dv <= 1024 && H <= 65535, "spy_mlstm: heads of %d x %d (key size up to 256, value size up to 1024)", d, dv);
     SPY_REQUIRE(cap > 0.f, "spy_mlstm: the gates' cap must be positive");
-    const dim3 grid(S, H);
-    SPY_DISPATCH(dtype, TA, SPY_DISPATCH(w_dtype, TW, MM_LAUNCH(mlstm_kernel, (TA*)out, state, (const TA*)x, xs, q_off, k_off, v_off,
-        g_off, gates, (const TW*)bi, (const TW*)bf, cap, (const TW*)norm_w, eps, cu_q, slot_ids, num_slots, H, d, dv)));
+    const int NS = (dv + MM_SLICE - 1) / MM_SLICE;
+    const dim3 grid(S, H, NS);
+    SPY_DISPATCH(dtype, TA, SPY_DISPATCH(w_dtype, TW, MM_LAUNCH(mlstm_kernel, o_tmp, state, (const TA*)x, xs, q_off, k_off, v_off, gates,
+        (const TW*)bi, (const TW*)bf, cap, cu_q, slot_ids, num_slots, H, d, dv, NS)));
     SPY_CHECK_LAUNCH("spy_mlstm");
+    const dim3 ngrid(T, H);
+    const int nthreads = dv >= 256 ? 256 : 64;
+    SPY_DISPATCH(dtype, TA, SPY_DISPATCH(w_dtype, TW, (head_norm_gate_kernel<TA, TW><<<ngrid, nthreads, 0, st>>>(
+        (TA*)out, o_tmp, (const TA*)x + g_off, xs, (const TW*)norm_w, 1, eps, H, dv))));
+    SPY_CHECK_LAUNCH("spy_mlstm (norm and gate)");
     return 0;
 }
 
@@ -201,87 +238,120 @@ extern "C" int spy_causal_conv_silu(void* y, const void* x, long long xs, int dt
 // qkv [T, 2 G d + H dv]: the convolved, activated q (G heads of d), k (G heads of d), v (H heads of dv).  beta_pre [T, H]
 // and dec_pre [T, H d] float32: raw products.  gate: rows of H dv values, gs apart.  state [slots][stride]: S of head h at
 // h d dv, row dd and column j at dd dv + j.
-template <typename TA, typename TW, int DR, int BT>
-__global__ __launch_bounds__(BT) void delta_rule_kernel(
-    TA* __restrict__ out, float* __restrict__ state, long long state_stride, const TA* __restrict__ qkv, const float* __restrict__ beta_pre,
-    const float* __restrict__ dec_pre, const TW* __restrict__ a_log, const TW* __restrict__ dt_bias, const TA* __restrict__ gate,
-    long long gs, const TW* __restrict__ norm_w, float eps, const int* __restrict__ cu_q, const int* __restrict__ slot_ids, int num_slots,
-    int H, int G, int d, int dv) {
-    __shared__ float ks[DR], qs[DR], dec[DR], red1[32], red2[32];
-    const int s = blockIdx.x, h = blockIdx.y, j = threadIdx.x;
+template <typename TA, typename TW, int DR>
+__global__ __launch_bounds__(MM_SLICE) void delta_rule_kernel(
+    float* __restrict__ o_out, float* __restrict__ state, long long state_stride, const TA* __restrict__ qkv, const float* __restrict__ beta_pre,
+    const float* __restrict__ dec_pre, const TW* __restrict__ a_log, const TW* __restrict__ dt_bias, const int* __restrict__ cu_q,
+    const int* __restrict__ slot_ids, int num_slots, int H, int G, int d, int dv) {
+    __shared__ __align__(16) float ks[DR], qs[DR], dec[DR];
+    constexpr int R = DR / MM_SLICE;
+    const int s = blockIdx.x, h = blockIdx.y, c = blockIdx.z, lane = threadIdx.x;
+    const int j = c * MM_SLICE + lane;
     const int slot = slot_ids[s];
     if (slot < 0 || slot >= num_slots) return;
     const int g = h / (H / G);
     float* st = state + (size_t)slot * state_stride + (size_t)h * d * dv;
+    const bool col = j < dv;
     float S[DR];
-    const bool col = j < dv, row = j < d;
 #pragma unroll
     for (int dd = 0; dd < DR; ++dd) S[dd] = (col && dd < d) ? st[(size_t)dd * dv + j] : 0.f;
     const float rate = expf(to_f32<TW>(a_log[h]));
-    const float dtb = row ? to_f32<TW>(dt_bias[(size_t)h * d + j]) : 0.f;
-    const float wn = col ? to_f32<TW>(norm_w[j]) : 0.f;
+    float dtb[R];
+#pragma unroll
+    for (int i = 0; i < R; ++i) {
+        const int idx = lane + MM_SLICE * i;
+        dtb[i] = idx < d ? to_f32<TW>(dt_bias[(size_t)h * d + idx]) : 0.f;
+        ks[idx] = 0.f;
+        qs[idx] = 0.f;
+        dec[idx] = 1.f;
+    }
     const float qscale = 1.0f / sqrtf((float)d);
     const int C = 2 * G * d + H * dv;
-    const int t1 = cu_q[s + 1];
-    for (int t = cu_q[s]; t < t1; ++t) {
-        const TA* xr = qkv + (size_t)t * C;
-        float qq = 0.f, kk = 0.f, dc = 1.f;
-        if (row) {
-            qq = to_f32<TA>(xr[(size_t)g * d + j]);
-            kk = to_f32<TA>(xr[(size_t)(G + g) * d + j]);
-            const float z = dec_pre[(size_t)t * H * d + (size_t)h * d + j] + dtb;
-            dc = expf(-rate * softplus_f(z));
+    const int t0 = cu_q[s], t1 = cu_q[s + 1];
+    float kc[R], qc[R], zc[R], vc = 0.f, bc = 0.f;
+    float kn[R], qn[R], zn[R], vn = 0.f, bn = 0.f;
+#define DELTA_LOAD(K, Q, Z, V, B, TT)                                                          \
+    {                                                                                          \
+        const TA* xr_ = qkv + (size_t)(TT) * C;                                                \
+        _Pragma("unroll") for (int i = 0; i < R; ++i) {                                        \
+            const int idx = lane + MM_SLICE * i;                                               \
+            Q[i] = idx < d ? to_f32<TA>(xr_[(size_t)g * d + idx]) : 0.f;                       \
+            K[i] = idx < d ? to_f32<TA>(xr_[(size_t)(G + g) * d + idx]) : 0.f;                 \
+            Z[i] = idx < d ? dec_pre[((size_t)(TT) * H + h) * d + idx] : 0.f;                  \
+        }                                                                                      \
+        V = col ? to_f32<TA>(xr_[(size_t)2 * G * d + (size_t)h * dv + j]) : 0.f;               \
+        B = beta_pre[(size_t)(TT) * H + h];                                                    \
+    }
+    if (t0 < t1) DELTA_LOAD(kc, qc, zc, vc, bc, t0)
+    for (int t = t0; t < t1; ++t) {
+        if (t + 1 < t1) DELTA_LOAD(kn, qn, zn, vn, bn, t + 1)
+        float sq = 0.f, sk = 0.f;
+#pragma unroll
+        for (int i = 0; i < R; ++i) { sq = fmaf(qc[i], qc[i], sq); sk = fmaf(kc[i], kc[i], sk); }
+        sq = wave_sum(sq);
+        sk = wave_sum(sk);
+        const float rq = qscale / sqrtf(sq + 1e-6f), rk = 1.0f / sqrtf(sk + 1e-6f);
+#pragma unroll
+        for (int i = 0; i < R; ++i) {
+            const int idx = lane + MM_SLICE * i;
+            if (idx < d) {
+                qs[idx] = qc[i] * rq;
+                ks[idx] = kc[i] * rk;
+                dec[idx] = expf(-rate * softplus_f(zc[i] + dtb[i]));
+            }
         }
-        const float vj = col ? to_f32<TA>(xr[(size_t)2 * G * d + (size_t)h * dv + j]) : 0.f;
-        const float gj = col ? to_f32<TA>(gate[(size_t)t * gs + (size_t)h * dv + j]) : 0.f;
-        const float beta = mm_sigmoid(beta_pre[(size_t)t * H + h]);
-        float sq = qq * qq, sk = kk * kk;
-        block_sum2(sq, sk, red1);
-        if (row) {
-            qs[j] = qq / sqrtf(sq + 1e-6f) * qscale;
-            ks[j] = kk / sqrtf(sk + 1e-6f);
-            dec[j] = dc;
-        }
+        const float beta = mm_sigmoid(bc);
         __syncthreads();
         float r = 0.f;
 #pragma unroll
-        for (int dd = 0; dd < DR; ++dd) {
+        for (int dd = 0; dd < DR; dd += 4) {
             if (dd < d) {
-                S[dd] *= dec[dd];
-                r = fmaf(S[dd], ks[dd], r);
+                const float4 k4 = *reinterpret_cast<const float4*>(ks + dd), g4 = *reinterpret_cast<const float4*>(dec + dd);
+                S[dd] *= g4.x;     r = fmaf(S[dd], k4.x, r);
+                S[dd + 1] *= g4.y; r = fmaf(S[dd + 1], k4.y, r);
+                S[dd + 2] *= g4.z; r = fmaf(S[dd + 2], k4.z, r);
+                S[dd + 3] *= g4.w; r = fmaf(S[dd + 3], k4.w, r);
             }
         }
-        const float u = beta * (vj - r);
+        const float u = beta * (vc - r);
         float acc = 0.f;
 #pragma unroll
-        for (int dd = 0; dd < DR; ++dd) {
+        for (int dd = 0; dd < DR; dd += 4) {
             if (dd < d) {
-                S[dd] = fmaf(ks[dd], u, S[dd]);
-                acc = fmaf(S[dd], qs[dd], acc);
+                const float4 k4 = *reinterpret_cast<const float4*>(ks + dd), q4 = *reinterpret_cast<const float4*>(qs + dd);
+                S[dd] = fmaf(k4.x, u, S[dd]);         acc = fmaf(S[dd], q4.x, acc);
+                S[dd + 1] = fmaf(k4.y, u, S[dd + 1]); acc = fmaf(S[dd + 1], q4.y, acc);
+                S[dd + 2] = fmaf(k4.z, u, S[dd + 2]); acc = fmaf(S[dd + 2], q4.z, acc);
+                S[dd + 3] = fmaf(k4.w, u, S[dd + 3]); acc = fmaf(S[dd + 3], q4.w, acc);
             }
         }
-        float ss = col ? acc * acc : 0.f, unused = 0.f;
-        block_sum2(ss, unused, red2);
-        if (col) {
-            const float rr = 1.0f / sqrtf(ss / (float)dv + eps);
-            out[(size_t)t * H * dv + (size_t)h * dv + j] = from_f32<TA>(((acc * rr) * wn) * mm_sigmoid(gj));
-        }
+        if (col) o_out[((size_t)t * H + h) * dv + j] = acc;
+        __syncthreads();
+#pragma unroll
+        for (int i = 0; i < R; ++i) { kc[i] = kn[i]; qc[i] = qn[i]; zc[i] = zn[i]; }
+        vc = vn; bc = bn;
     }
+#undef DELTA_LOAD
 #pragma unroll
     for (int dd = 0; dd < DR; ++dd)
         if (col && dd < d) st[(size_t)dd * dv + j] = S[dd];
 }
 
-extern "C" int spy_delta_rule(void* out, float* state, long long state_stride, const void* qkv, int dtype, const float* beta_pre,
+extern "C" int spy_delta_rule(void* out, float* o_tmp, float* state, long long state_stride, const void* qkv, int dtype, const float* beta_pre,
                               const float* dec_pre, const void* a_log, const void* dt_bias, int w_dtype, const void* gate, long long gs,
                               const void* norm_w, float eps, const int* cu_q, const int* slot_ids, int num_slots, int S, int T, int H,
                               int G, int d, int dv, hipStream_t st) {
-    SPY_REQUIRE(S > 0 && T > 0 && H > 0 && G > 0 && H % G == 0 && d > 0 && dv > 0 && num_slots > 0, "spy_delta_rule: empty operand");
+    SPY_REQUIRE(S > 0 && T > 0 && H > 0 && G > 0 && H % G == 0 && d > 0 && dv > 0 && num_slots > 0 && o_tmp, "spy_delta_rule: empty operand");
     SPY_REQUIRE(d <= 256 && dv <= 1024 && H <= 65535, "spy_delta_rule: heads of %d x %d (key size up to 256, value size up to 1024)", d, dv);
     SPY_REQUIRE(state_stride >= (long long)H * d * dv && gs >= (long long)H * dv, "spy_delta_rule: the state or the gate rows are too short");
-    const dim3 grid(S, H);
-    SPY_DISPATCH(dtype, TA, SPY_DISPATCH(w_dtype, TW, MM_LAUNCH(delta_rule_kernel, (TA*)out, state, state_stride, (const TA*)qkv, beta_pre,
-        dec_pre, (const TW*)a_log, (const TW*)dt_bias, (const TA*)gate, gs, (const TW*)norm_w, eps, cu_q, slot_ids, num_slots, H, G, d, dv)));
+    const dim3 grid(S, H, (dv + MM_SLICE - 1) / MM_SLICE);
+    SPY_DISPATCH(dtype, TA, SPY_DISPATCH(w_dtype, TW, MM_LAUNCH(delta_rule_kernel, o_tmp, state, state_stride, (const TA*)qkv, beta_pre,
+        dec_pre, (const TW*)a_log, (const TW*)dt_bias, cu_q, slot_ids, num_slots, H, G, d, dv)));
     SPY_CHECK_LAUNCH("spy_delta_rule");
+    const dim3 ngrid(T, H);
+    const int nthreads = dv >= 256 ? 256 : 64;
+    SPY_DISPATCH(dtype, TA, SPY_DISPATCH(w_dtype, TW, (head_norm_gate_kernel<TA, TW><<<ngrid, nthreads, 0, st>>>(
+        (TA*)out, o_tmp, (const TA*)gate, gs, (const TW*)norm_w, 0, eps, H, dv))));
+    SPY_CHECK_LAUNCH("spy_delta_rule (norm and gate)");
     return 0;
 }

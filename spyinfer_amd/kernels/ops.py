@@ -1192,6 +1192,13 @@ def sigmoid_gate(y: torch.Tensor, gate: torch.Tensor) -> torch.Tensor:
 # --------------------------------------------------------------------------
 # Recurrent mixers with a matrix state per head
 MATRIX_MEMORY_MAX_DIM, MATRIX_MEMORY_MAX_VDIM = 256, 1024
+MATRIX_MEMORY_SLICE = 64          # value channels that one wave of the recurrences owns
+
+
+def mlstm_state_size(H: int, d: int, dv: int) -> int:
+    """float32 values of one request's mLSTM state: per head S [d, dv], then n [d] and the running maximum once for every
+    slice of value channels (the slices' waves each keep their own copy)."""
+    return H * (d * dv + -(-dv // MATRIX_MEMORY_SLICE) * (d + 1))
 
 
 def _entries(cu_q: torch.Tensor, slot_ids: torch.Tensor, what: str) -> int:
@@ -1206,8 +1213,8 @@ def mlstm(x: torch.Tensor, q_off: int, k_off: int, v_off: int, g_off: int, gates
     """The mLSTM recurrence over the step's tokens.  ``x``: rows of the fused projection with q (H heads of d) at column
     ``q_off``, k at ``k_off``, v (H heads of dv) at ``v_off`` and the output gate's rows at ``g_off``; ``gates [T, 2 H]``
     float32: the raw products of the input and forget gates (their biases ``bi``, ``bf [H]``; both capped by
-    cap tanh(. / cap)); ``state [slots, H (d dv + d + 1)]`` float32 holds S, n and the running maximum of every head, read
-    at an entry's start and left at its end.  Returns [T, H dv]: each head's read-out over its root mean square, times
+    cap tanh(. / cap)); ``state [slots, mlstm_state_size(H, d, dv)]`` float32 holds S, n and the running maximum of every
+    head, read at an entry's start and left at its end.  Returns [T, H dv]: each head's read-out over its root mean square, times
     ``norm_w``, times sigmoid(gate)."""
     xs = _row_view(x, "mlstm")
     T = x.shape[0]
@@ -1220,10 +1227,12 @@ def mlstm(x: torch.Tensor, q_off: int, k_off: int, v_off: int, g_off: int, gates
     _check(gates.dtype == torch.float32 and gates.shape == (T, 2 * H), "mlstm: the gates' products must be float32 [T, 2 H]")
     _check(bi.shape == (H,) and bf.shape == (H,) and norm_w.shape == (H * dv,) and bi.dtype == bf.dtype == norm_w.dtype,
            "mlstm: gate biases [H] and a norm weight [H dv] of one dtype expected")
-    _check(state.dtype == torch.float32 and state.dim() == 2 and state.shape[1] == H * (d * dv + d + 1), "mlstm: state must be float32 [slots, H (d dv + d + 1)]")
+    _check(state.dtype == torch.float32 and state.dim() == 2 and state.shape[1] == mlstm_state_size(H, d, dv),
+           "mlstm: state must be float32 [slots, mlstm_state_size(H, d, dv)]")
     out = torch.empty((T, H * dv), dtype=x.dtype, device=x.device)
     if T:
-        hip().call("spy_mlstm", _ptr(out), _ptr(state), ctypes.c_void_p(x.data_ptr()), ctypes.c_longlong(xs), _code(x, "x"), ctypes.c_int(q_off),
+        tmp = torch.empty((T, H * dv), dtype=torch.float32, device=x.device)        # the read-outs before the heads' norm
+        hip().call("spy_mlstm", _ptr(out), _ptr(tmp), _ptr(state), ctypes.c_void_p(x.data_ptr()), ctypes.c_longlong(xs), _code(x, "x"), ctypes.c_int(q_off),
                    ctypes.c_int(k_off), ctypes.c_int(v_off), ctypes.c_int(g_off), _ptr(gates), _ptr(bi), _ptr(bf), _code(bi, "gate biases"),
                    ctypes.c_float(cap), _ptr(norm_w), ctypes.c_float(eps), _ptr(cu_q), _ptr(slot_ids), ctypes.c_int(state.shape[0]),
                    ctypes.c_int(S), ctypes.c_int(T), ctypes.c_int(H), ctypes.c_int(d), ctypes.c_int(dv), _Hip.stream())
@@ -1277,7 +1286,8 @@ def delta_rule(qkv: torch.Tensor, beta_pre: torch.Tensor, dec_pre: torch.Tensor,
     _check(state.dtype == torch.float32 and state.dim() == 2 and state.shape[1] >= H * d * dv, "delta_rule: state must be float32 [slots, >= H d dv]")
     out = torch.empty((T, H * dv), dtype=qkv.dtype, device=qkv.device)
     if T:
-        hip().call("spy_delta_rule", _ptr(out), _ptr(state), ctypes.c_longlong(state.shape[1]), _ptr(qkv), _code(qkv, "qkv"), _ptr(beta_pre),
+        tmp = torch.empty((T, H * dv), dtype=torch.float32, device=qkv.device)      # the read-outs before the heads' norm
+        hip().call("spy_delta_rule", _ptr(out), _ptr(tmp), _ptr(state), ctypes.c_longlong(state.shape[1]), _ptr(qkv), _code(qkv, "qkv"), _ptr(beta_pre),
                    _ptr(dec_pre), _ptr(a_log), _ptr(dt_bias), _code(a_log, "decay numbers"), ctypes.c_void_p(gate.data_ptr()), ctypes.c_longlong(gs),
                    _ptr(norm_w), ctypes.c_float(eps), _ptr(cu_q), _ptr(slot_ids), ctypes.c_int(state.shape[0]), ctypes.c_int(S), ctypes.c_int(T),
                    ctypes.c_int(H), ctypes.c_int(G), ctypes.c_int(d), ctypes.c_int(dv), _Hip.stream())

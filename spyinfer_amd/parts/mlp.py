@@ -114,8 +114,9 @@ class MoEMLP(FeedForward):
 
     def bind(self, prefix, weights):
         router, corr, gate, up, down = (prefix + "." + n for n in self.names)
-        # the router and its correction are float32 whatever the run: its scores decide, they are not activations
-        self.w_router = weights.pop(router).float().contiguous()
+        # the router's product keeps its float32 sums (bfloat16 operands multiply exactly in float32), and everything
+        # behind it is float32: its scores decide, they are not activations
+        self.w_router = weights.pop(router)
         self.correction = weights[corr].float().contiguous()
         E = self.experts
         mats = [weights.pop(n % e) for e in range(E) for n in (gate, up, down)]

@@ -120,8 +120,10 @@ class MLSTM(Mixer):
         # recurrence's exponentials, come from a second, small product whose result stays float32
         self.w_in, self.w_in_tiled = ops.weight_forms(torch.cat(mats, dim=0).contiguous())
         del mats
-        # (kept float32: a product of a few rows of any shape, through the true 32-bit kernel in both runs)
-        self.w_gates = torch.cat([weights.pop(i).float(), weights.pop(f).float()], dim=0).contiguous()
+        gi, gf = weights.pop(i), weights.pop(f)
+        if gi.dtype != gf.dtype:
+            gi, gf = gi.float(), gf.float()
+        self.w_gates = torch.cat([gi, gf], dim=0).contiguous()
         self.w_o, self.w_o_tiled = ops.weight_forms(weights.pop(o))
         small = [weights[ib], weights[fb], weights[norm]]
         if len({t.dtype for t in small}) > 1:
@@ -129,8 +131,7 @@ class MLSTM(Mixer):
         self.b_i, self.b_f, self.norm = small
 
     def cache_spec(self):
-        H, d, dv = self.heads, self.dim, self.vdim
-        return FixedState((H * (d * dv + d + 1),), "float32")
+        return FixedState((ops.mlstm_state_size(self.heads, self.dim, self.vdim),), "float32")
 
     def capturable(self, batch):
         return True
@@ -186,8 +187,11 @@ class ChannelDelta(Mixer):
         # recurrence's exponentials (beta, the decay's inner projection) comes from a second product that stays float32
         self.w_in, self.w_in_tiled = ops.weight_forms(torch.cat(mats, dim=0).contiguous())
         del mats
-        self.w_small = torch.cat([weights.pop(b).float(), weights.pop(a1).float()], dim=0).contiguous()
-        self.w_a2 = weights.pop(a2).float().contiguous()
+        small = [weights.pop(b), weights.pop(a1)]
+        if small[0].dtype != small[1].dtype:
+            small = [t.float() for t in small]
+        self.w_small = torch.cat(small, dim=0).contiguous()
+        self.w_a2 = weights.pop(a2)
         self.w_g2, self.w_g2_tiled = ops.weight_forms(weights.pop(g2))
         self.w_o, self.w_o_tiled = ops.weight_forms(weights.pop(o))
         taps = [weights[n] for n in (qc, kc, vc)]
@@ -209,9 +213,10 @@ class ChannelDelta(Mixer):
             raise ValueError("a recurrence cannot run on another layer's state without writing it")
         H, G, d, dv, C = self.heads, self.kv_heads, self.dim, self.vdim, self._channels()
         proj = ops.linear_few(x, self.w_in, self.w_in_tiled)
-        small = ops.linear(x, self.w_small, torch.float32)                    # [beta | a1], float32
+        small = ops.linear(x, self.w_small, torch.float32)                    # [beta | a1], float32 sums kept
         beta_pre = small[:, :H].contiguous()
-        dec_pre = ops.linear(small[:, H:].contiguous(), self.w_a2, torch.float32)
+        # (the inner projection's result is an activation: it takes the activation dtype on its way into the outer one)
+        dec_pre = ops.linear(small[:, H:].to(self.w_a2.dtype).contiguous(), self.w_a2, torch.float32)
         gate = ops.linear_few(proj[:, C:].contiguous(), self.w_g2, self.w_g2_tiled)
         cu_q, slots = batch.array("cu_q"), batch.array("slot_ids")
         qkv = ops.causal_conv_silu(proj[:, :C], self.taps, cache.state, H * d * dv, batch.array("token_entry"), cu_q, slots)

@@ -247,9 +247,9 @@ class EmuOps:
         f = x.float()
         out = torch.zeros((T, H, dv), dtype=torch.float32)
         for s in range(slot_ids.shape[0]):
-            st = state[int(slot_ids[s])].view(H, d * dv + d + 1)
+            st = state[int(slot_ids[s])].view(H, -1)          # per head: S, then (n, m) once per slice of value channels
             for h in range(H):
-                S, n, m = st[h, :d * dv].view(d, dv).clone(), st[h, d * dv:d * dv + d].clone(), float(st[h, -1])
+                S, n, m = st[h, :d * dv].view(d, dv).clone(), st[h, d * dv:d * dv + d].clone(), float(st[h, d * dv + d])
                 for t in range(int(cu_q[s]), int(cu_q[s + 1])):
                     q = f[t, q_off + h * d:q_off + (h + 1) * d] * d ** -0.5
                     k = f[t, k_off + h * d:k_off + (h + 1) * d]
@@ -264,8 +264,9 @@ class EmuOps:
                     den = max(abs(float(n @ q)), float(torch.exp(torch.tensor(-m)))) + 1e-6
                     out[t, h] = (S.T @ q) / den
                 st[h, :d * dv] = S.reshape(-1)
-                st[h, d * dv:d * dv + d] = n
-                st[h, -1] = m
+                for c in range((st.shape[1] - d * dv) // (d + 1)):
+                    st[h, d * dv + c * (d + 1):d * dv + c * (d + 1) + d] = n
+                    st[h, d * dv + c * (d + 1) + d] = m
         out = out * torch.rsqrt((out * out).mean(-1, keepdim=True) + eps)
         g = f[:, g_off:g_off + H * dv]
         return (out.reshape(T, H * dv) * norm_w.float() * torch.sigmoid(g)).to(x.dtype)

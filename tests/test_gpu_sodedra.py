@@ -99,7 +99,7 @@ def test_mlstm_carries_its_state_between_steps(dtype, H, d, dv):
     proj = rnd(g, T, 2 * H * d + 2 * H * dv).to(DT[dtype])
     gates = rnd(g, T, 2 * H, std=3.0).float()
     bi, bf, nw = rnd(g, H).to(DT[dtype]), (rnd(g, H) + 2.0).to(DT[dtype]), (1.0 + rnd(g, H * dv, std=0.2)).to(DT[dtype])
-    state = torch.full((4, H * (d * dv + d + 1)), float("nan"), device=dev)
+    state = torch.full((4, ops.mlstm_state_size(H, d, dv)), float("nan"), device=dev)
     state[[2, 0, 3]] = 0.0
     got = torch.zeros((T, H * dv), dtype=torch.float64)
     for rows, cu, sl, _ in two_steps(lengths, cut):

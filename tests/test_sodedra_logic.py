@@ -51,7 +51,7 @@ def test_cache_kinds_follow_the_layers():
     specs = model.cache_specs()
     # key and value heads of different sizes share one padded head size; windows give pages back, recurrences keep slots
     assert specs[0] == PagedKV(2, 16, 9) and specs[3] == PagedKV(1, 16, None) and specs[6] == PagedKV(3, 4, 5)
-    assert specs[1] == FixedState((3 * (5 * 7 + 5 + 1),), "float32")
+    assert specs[1] == FixedState((3 * (5 * 7 + 5 + 1),), "float32")          # (seven value channels: one slice)
     assert specs[2] == FixedState((4 * 6 * 5 + 2 * (2 * 2 * 6 + 4 * 5),), "float32")
     assert model.lm_head.tied_to is model.embed
 
