@@ -38,14 +38,26 @@ __global__ void head_norm_gate_kernel(TA* __restrict__ out, const float* __restr
 }
 
 // ---- mLSTM ----------------------------------------------------------------------------------------------------------
+// In place over the gates' raw products [T, 2 H]: the capped log gates i = cap tanh((. + bi) / cap) and
+// f = logsigmoid(cap tanh((. + bf) / cap)), for all tokens at once (the walk below has only the running maximum left).
+template <typename TW>
+__global__ void mlstm_gates_kernel(float* __restrict__ gates, const TW* __restrict__ bi, const TW* __restrict__ bf, float cap, int T, int H) {
+    const size_t total = (size_t)T * 2 * H;
+    for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < total; i += (size_t)gridDim.x * blockDim.x) {
+        const int c = (int)(i % (2 * H));
+        if (c < H) gates[i] = cap * tanhf((gates[i] + to_f32<TW>(bi[c])) / cap);
+        else gates[i] = mm_logsigmoid(cap * tanhf((gates[i] + to_f32<TW>(bf[c - H])) / cap));
+    }
+}
+
 // x: rows of the fused projection, xs values apart; q at column q_off (H heads of d), k at k_off, v at v_off (H heads of
-// dv).  gates [T, 2 H] float32: the raw products of the input and the forget gate.  state [slots][H][d dv + NS (d + 1)]:
+// dv).  gates [T, 2 H] float32: the log input and forget gates (mlstm_gates_kernel).  state [slots][H][d dv + NS (d + 1)]:
 // S (row dd, column j at dd dv + j), then for every slice of 64 columns its own copy of n and m (the slices' waves do
 // not wait for each other, so none may read what another has already moved on).
 template <typename TA, typename TW, int DR>
 __global__ __launch_bounds__(MM_SLICE) void mlstm_kernel(
     float* __restrict__ o_out, float* __restrict__ state, const TA* __restrict__ x, long long xs, int q_off, int k_off, int v_off,
-    const float* __restrict__ gates, const TW* __restrict__ bi, const TW* __restrict__ bf, float cap, const int* __restrict__ cu_q,
+    const float* __restrict__ gates, const int* __restrict__ cu_q,
     const int* __restrict__ slot_ids, int num_slots, int H, int d, int dv, int NS) {
     __shared__ __align__(16) float ks[DR], qs[DR];
     constexpr int R = DR / MM_SLICE;
@@ -69,7 +81,6 @@ __global__ __launch_bounds__(MM_SLICE) void mlstm_kernel(
         qs[idx] = 0.f;
     }
     float m = nm[d];
-    const float b_i = to_f32<TW>(bi[h]), b_f = to_f32<TW>(bf[h]);
     const float qscale = 1.0f / sqrtf((float)d);
     const int t0 = cu_q[s], t1 = cu_q[s + 1];
     float kc[R], qc[R], vc = 0.f, gic = 0.f, gfc = 0.f;
@@ -94,8 +105,7 @@ __global__ __launch_bounds__(MM_SLICE) void mlstm_kernel(
             const int idx = lane + MM_SLICE * i;
             if (idx < d) { ks[idx] = kc[i]; qs[idx] = qc[i]; }
         }
-        const float ig = cap * tanhf((gic + b_i) / cap);
-        const float fg = mm_logsigmoid(cap * tanhf((gfc + b_f) / cap));
+        const float ig = gic, fg = gfc;
         const float m_new = fmaxf(fg + m, ig);
         const float a = expf(fg + m - m_new), b = expf(ig - m_new);
         m = m_new;
@@ -146,15 +156,21 @@ __global__ __launch_bounds__(MM_SLICE) void mlstm_kernel(
     } while (0)
 
 extern "C" int spy_mlstm(void* out, float* o_tmp, float* state, const void* x, long long xs, int dtype, int q_off, int k_off, int v_off,
-                         int g_off, const float* gates, const void* bi, const void* bf, int w_dtype, float cap, const void* norm_w,
+                         int g_off, float* gates, const void* bi, const void* bf, int w_dtype, float cap, const void* norm_w,
                          float eps, const int* cu_q, const int* slot_ids, int num_slots, int S, int T, int H, int d, int dv, hipStream_t st) {
     SPY_REQUIRE(S > 0 && T > 0 && H > 0 && d > 0 && dv > 0 && num_slots > 0 && o_tmp, "spy_mlstm: empty operand");
     SPY_REQUIRE(d <= 256 && dv <= 1024 && H <= 65535, "spy_mlstm: heads of %d x %d (key size up to 256, value size up to 1024)", d, dv);
     SPY_REQUIRE(cap > 0.f, "spy_mlstm: the gates' cap must be positive");
     const int NS = (dv + MM_SLICE - 1) / MM_SLICE;
     const dim3 grid(S, H, NS);
+    {
+        const size_t total = (size_t)T * 2 * H;
+        const unsigned blocks = (unsigned)((total + 255) / 256 > 4096 ? 4096 : (total + 255) / 256);
+        SPY_DISPATCH(w_dtype, TW, (mlstm_gates_kernel<TW><<<blocks, 256, 0, st>>>(gates, (const TW*)bi, (const TW*)bf, cap, T, H)));
+        SPY_CHECK_LAUNCH("spy_mlstm (gates)");
+    }
     SPY_DISPATCH(dtype, TA, SPY_DISPATCH(w_dtype, TW, MM_LAUNCH(mlstm_kernel, o_tmp, state, (const TA*)x, xs, q_off, k_off, v_off, gates,
-        (const TW*)bi, (const TW*)bf, cap, cu_q, slot_ids, num_slots, H, d, dv, NS)));
+        cu_q, slot_ids, num_slots, H, d, dv, NS)));
     SPY_CHECK_LAUNCH("spy_mlstm");
     const dim3 ngrid(T, H);
     const int nthreads = dv >= 256 ? 256 : 64;
@@ -238,10 +254,46 @@ extern "C" int spy_causal_conv_silu(void* y, const void* x, long long xs, int dt
 // qkv [T, 2 G d + H dv]: the convolved, activated q (G heads of d), k (G heads of d), v (H heads of dv).  beta_pre [T, H]
 // and dec_pre [T, H d] float32: raw products.  gate: rows of H dv values, gs apart.  state [slots][stride]: S of head h at
 // h d dv, row dd and column j at dd dv + j.
+// For all tokens at once, one wave per (token, unit): units 0 .. G - 1 turn head g's q and k into unit vectors (q also
+// times d^-1/2) in qk [T, 2 G d] float32; units G .. G + H - 1 turn head h's raw decay products into the decays
+// exp(-exp(a_log) softplus(. + dt_bias)) and its raw beta product into sigmoid(.), both in place.
+template <typename TA, typename TW>
+__global__ __launch_bounds__(64) void delta_prepare_kernel(float* __restrict__ qk, const TA* __restrict__ qkv, float* __restrict__ beta,
+                                                          float* __restrict__ dec, const TW* __restrict__ a_log,
+                                                          const TW* __restrict__ dt_bias, int H, int G, int d, int dv) {
+    const int t = blockIdx.x, unit = blockIdx.y, lane = threadIdx.x;
+    const int C = 2 * G * d + H * dv;
+    if (unit < G) {
+        const TA* q = qkv + (size_t)t * C + (size_t)unit * d;
+        const TA* k = qkv + (size_t)t * C + (size_t)(G + unit) * d;
+        float sq = 0.f, sk = 0.f;
+        for (int i = lane; i < d; i += 64) {
+            const float a = to_f32<TA>(q[i]), b = to_f32<TA>(k[i]);
+            sq = fmaf(a, a, sq);
+            sk = fmaf(b, b, sk);
+        }
+        sq = wave_sum(sq);
+        sk = wave_sum(sk);
+        const float rq = 1.0f / sqrtf(sq + 1e-6f) / sqrtf((float)d), rk = 1.0f / sqrtf(sk + 1e-6f);
+        float* oq = qk + (size_t)t * 2 * G * d + (size_t)unit * d;
+        float* ok = qk + (size_t)t * 2 * G * d + (size_t)(G + unit) * d;
+        for (int i = lane; i < d; i += 64) {
+            oq[i] = to_f32<TA>(q[i]) * rq;
+            ok[i] = to_f32<TA>(k[i]) * rk;
+        }
+        return;
+    }
+    const int h = unit - G;
+    const float rate = expf(to_f32<TW>(a_log[h]));
+    float* z = dec + ((size_t)t * H + h) * d;
+    for (int i = lane; i < d; i += 64) z[i] = expf(-rate * softplus_f(z[i] + to_f32<TW>(dt_bias[(size_t)h * d + i])));
+    if (lane == 0) beta[(size_t)t * H + h] = mm_sigmoid(beta[(size_t)t * H + h]);
+}
+
 template <typename TA, typename TW, int DR>
 __global__ __launch_bounds__(MM_SLICE) void delta_rule_kernel(
-    float* __restrict__ o_out, float* __restrict__ state, long long state_stride, const TA* __restrict__ qkv, const float* __restrict__ beta_pre,
-    const float* __restrict__ dec_pre, const TW* __restrict__ a_log, const TW* __restrict__ dt_bias, const int* __restrict__ cu_q,
+    float* __restrict__ o_out, float* __restrict__ state, long long state_stride, const TA* __restrict__ qkv, const float* __restrict__ qk,
+    const float* __restrict__ beta_pre, const float* __restrict__ dec_pre, const int* __restrict__ cu_q,
     const int* __restrict__ slot_ids, int num_slots, int H, int G, int d, int dv) {
     __shared__ __align__(16) float ks[DR], qs[DR], dec[DR];
     constexpr int R = DR / MM_SLICE;
@@ -255,17 +307,13 @@ __global__ __launch_bounds__(MM_SLICE) void delta_rule_kernel(
     float S[DR];
 #pragma unroll
     for (int dd = 0; dd < DR; ++dd) S[dd] = (col && dd < d) ? st[(size_t)dd * dv + j] : 0.f;
-    const float rate = expf(to_f32<TW>(a_log[h]));
-    float dtb[R];
 #pragma unroll
     for (int i = 0; i < R; ++i) {
         const int idx = lane + MM_SLICE * i;
-        dtb[i] = idx < d ? to_f32<TW>(dt_bias[(size_t)h * d + idx]) : 0.f;
         ks[idx] = 0.f;
         qs[idx] = 0.f;
         dec[idx] = 1.f;
     }
-    const float qscale = 1.0f / sqrtf((float)d);
     const int C = 2 * G * d + H * dv;
     const int t0 = cu_q[s], t1 = cu_q[s + 1];
     float kc[R], qc[R], zc[R], vc = 0.f, bc = 0.f;
@@ -273,11 +321,12 @@ __global__ __launch_bounds__(MM_SLICE) void delta_rule_kernel(
 #define DELTA_LOAD(K, Q, Z, V, B, TT)                                                          \
     {                                                                                          \
         const TA* xr_ = qkv + (size_t)(TT) * C;                                                \
+        const float* qk_ = qk + (size_t)(TT) * 2 * G * d;                                      \
         _Pragma("unroll") for (int i = 0; i < R; ++i) {                                        \
             const int idx = lane + MM_SLICE * i;                                               \
-            Q[i] = idx < d ? to_f32<TA>(xr_[(size_t)g * d + idx]) : 0.f;                       \
-            K[i] = idx < d ? to_f32<TA>(xr_[(size_t)(G + g) * d + idx]) : 0.f;                 \
-            Z[i] = idx < d ? dec_pre[((size_t)(TT) * H + h) * d + idx] : 0.f;                  \
+            Q[i] = idx < d ? qk_[(size_t)g * d + idx] : 0.f;                                   \
+            K[i] = idx < d ? qk_[(size_t)(G + g) * d + idx] : 0.f;                             \
+            Z[i] = idx < d ? dec_pre[((size_t)(TT) * H + h) * d + idx] : 1.f;                  \
         }                                                                                      \
         V = col ? to_f32<TA>(xr_[(size_t)2 * G * d + (size_t)h * dv + j]) : 0.f;               \
         B = beta_pre[(size_t)(TT) * H + h];                                                    \
@@ -285,22 +334,16 @@ __global__ __launch_bounds__(MM_SLICE) void delta_rule_kernel(
     if (t0 < t1) DELTA_LOAD(kc, qc, zc, vc, bc, t0)
     for (int t = t0; t < t1; ++t) {
         if (t + 1 < t1) DELTA_LOAD(kn, qn, zn, vn, bn, t + 1)
-        float sq = 0.f, sk = 0.f;
-#pragma unroll
-        for (int i = 0; i < R; ++i) { sq = fmaf(qc[i], qc[i], sq); sk = fmaf(kc[i], kc[i], sk); }
-        sq = wave_sum(sq);
-        sk = wave_sum(sk);
-        const float rq = qscale / sqrtf(sq + 1e-6f), rk = 1.0f / sqrtf(sk + 1e-6f);
 #pragma unroll
         for (int i = 0; i < R; ++i) {
             const int idx = lane + MM_SLICE * i;
             if (idx < d) {
-                qs[idx] = qc[i] * rq;
-                ks[idx] = kc[i] * rk;
-                dec[idx] = expf(-rate * softplus_f(zc[i] + dtb[i]));
+                qs[idx] = qc[i];
+                ks[idx] = kc[i];
+                dec[idx] = zc[i];
             }
         }
-        const float beta = mm_sigmoid(bc);
+        const float beta = bc;
         __syncthreads();
         float r = 0.f;
 #pragma unroll
@@ -337,16 +380,21 @@ __global__ __launch_bounds__(MM_SLICE) void delta_rule_kernel(
         if (col && dd < d) st[(size_t)dd * dv + j] = S[dd];
 }
 
-extern "C" int spy_delta_rule(void* out, float* o_tmp, float* state, long long state_stride, const void* qkv, int dtype, const float* beta_pre,
-                              const float* dec_pre, const void* a_log, const void* dt_bias, int w_dtype, const void* gate, long long gs,
+extern "C" int spy_delta_rule(void* out, float* o_tmp, float* qk_tmp, float* state, long long state_stride, const void* qkv, int dtype,
+                              float* beta_pre, float* dec_pre, const void* a_log, const void* dt_bias, int w_dtype, const void* gate, long long gs,
                               const void* norm_w, float eps, const int* cu_q, const int* slot_ids, int num_slots, int S, int T, int H,
                               int G, int d, int dv, hipStream_t st) {
     SPY_REQUIRE(S > 0 && T > 0 && H > 0 && G > 0 && H % G == 0 && d > 0 && dv > 0 && num_slots > 0 && o_tmp, "spy_delta_rule: empty operand");
     SPY_REQUIRE(d <= 256 && dv <= 1024 && H <= 65535, "spy_delta_rule: heads of %d x %d (key size up to 256, value size up to 1024)", d, dv);
     SPY_REQUIRE(state_stride >= (long long)H * d * dv && gs >= (long long)H * dv, "spy_delta_rule: the state or the gate rows are too short");
+    SPY_REQUIRE(qk_tmp && G + H <= 65535, "spy_delta_rule: no room for the unit vectors");
+    const dim3 pgrid(T, G + H);
+    SPY_DISPATCH(dtype, TA, SPY_DISPATCH(w_dtype, TW, (delta_prepare_kernel<TA, TW><<<pgrid, 64, 0, st>>>(
+        qk_tmp, (const TA*)qkv, beta_pre, dec_pre, (const TW*)a_log, (const TW*)dt_bias, H, G, d, dv))));
+    SPY_CHECK_LAUNCH("spy_delta_rule (unit vectors and decays)");
     const dim3 grid(S, H, (dv + MM_SLICE - 1) / MM_SLICE);
-    SPY_DISPATCH(dtype, TA, SPY_DISPATCH(w_dtype, TW, MM_LAUNCH(delta_rule_kernel, o_tmp, state, state_stride, (const TA*)qkv, beta_pre,
-        dec_pre, (const TW*)a_log, (const TW*)dt_bias, cu_q, slot_ids, num_slots, H, G, d, dv)));
+    SPY_DISPATCH(dtype, TA, SPY_DISPATCH(w_dtype, TW, MM_LAUNCH(delta_rule_kernel, o_tmp, state, state_stride, (const TA*)qkv, qk_tmp, beta_pre,
+        dec_pre, cu_q, slot_ids, num_slots, H, G, d, dv)));
     SPY_CHECK_LAUNCH("spy_delta_rule");
     const dim3 ngrid(T, H);
     const int nthreads = dv >= 256 ? 256 : 64;

@@ -327,6 +327,119 @@ __global__ __launch_bounds__(256) void moe_gemm_mfma_kernel(TC* __restrict__ C, 
     }
 }
 
+
+// Many rows per expert: the same tiles, but the gathered rows of A go through LDS once per block and step of 128 of K
+// (the four waves read the same rows; loaded by each of them they swept the first-level cache), while every wave's W
+// fragments still come straight from memory, asked for before the block waits for the staged rows.
+#define MOE_ROWS 128                 // 8 row tiles
+#define MOE_LDS_STRIDE (128 + 8)     // values per staged row (16-byte pieces; the pad spreads the rows over the banks)
+template <bool GATED, typename TC>
+__global__ __launch_bounds__(256) void moe_gemm_mfma_lds_kernel(TC* __restrict__ C, const bf16_t* __restrict__ A, const bf16_t* __restrict__ W,
+                                                                const int* __restrict__ tile_expert, const int* __restrict__ sorted_pair,
+                                                                int gather, int max_tiles, int N, int K, long long w_stride) {
+    constexpr int MT = 8, NT = 2;
+    __shared__ __align__(16) bf16_t xs[MOE_ROWS * MOE_LDS_STRIDE];
+    __shared__ int src_row[MOE_ROWS];
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63;
+    const int r = lane & 15, g = lane >> 4;
+    const int n0 = (blockIdx.y * 4 + wave) * (GATED ? 16 : 32);
+    const bool cols = n0 < N;                        // (a wave without columns still helps to stage)
+    int t = blockIdx.x * MT;
+    const int t_end = min(t + MT, max_tiles);
+    const moe_bf16x8_t zero8 = {0, 0, 0, 0, 0, 0, 0, 0};
+    const int srow = threadIdx.x >> 4, spiece = threadIdx.x & 15;      // staging: rows srow + 16 i, 16-byte piece spiece
+    while (t < t_end) {
+        const int e = __builtin_amdgcn_readfirstlane(tile_expert[t]);
+        if (e < 0) break;
+        int run = 1;
+        while (t + run < t_end && __builtin_amdgcn_readfirstlane(tile_expert[t + run]) == e) ++run;
+        __syncthreads();                             // the run before has read its rows
+        if (threadIdx.x < MOE_ROWS) {
+            int src = -1;
+            if ((int)threadIdx.x < run * MOE_TM) {
+                const int row = t * MOE_TM + threadIdx.x;
+                const int p = sorted_pair[row];
+                src = p < 0 ? -1 : (gather > 0 ? p / gather : row);
+            }
+            src_row[threadIdx.x] = src;
+        }
+        __syncthreads();
+        int srcs[MT];
+#pragma unroll
+        for (int i = 0; i < MT; ++i) srcs[i] = src_row[srow + 16 * i];
+        bool xok[MT];
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt) xok[mt] = mt < run && src_row[mt * 16 + r] >= 0;
+        const bf16_t* We = W + (size_t)e * w_stride;
+        const bf16_t* wrow[NT];
+#pragma unroll
+        for (int nt = 0; nt < NT; ++nt) {
+            const int row = GATED ? nt * N + min(n0 + r, N - 1) : min(n0 + nt * 16 + r, N - 1);
+            wrow[nt] = We + (size_t)(cols ? row : 0) * K + 8 * g;
+        }
+        moe_f32x4_t acc[NT][MT];
+#pragma unroll
+        for (int nt = 0; nt < NT; ++nt)
+#pragma unroll
+            for (int mt = 0; mt < MT; ++mt) acc[nt][mt] = moe_f32x4_t{0.f, 0.f, 0.f, 0.f};
+        for (int k = 0; k < K; k += 128) {
+            moe_bf16x8_t a[NT][4];
+#pragma unroll
+            for (int j = 0; j < 4; ++j)
+#pragma unroll
+                for (int nt = 0; nt < NT; ++nt)
+                    a[nt][j] = (cols && k + 32 * j + 8 * g < K) ? *reinterpret_cast<const moe_bf16x8_t*>(wrow[nt] + k + 32 * j) : zero8;
+            moe_bf16x8_t stage[MT];
+            const bool kin = k + 8 * spiece < K;
+#pragma unroll
+            for (int i = 0; i < MT; ++i)
+                stage[i] = (i < run && srcs[i] >= 0 && kin) ? *reinterpret_cast<const moe_bf16x8_t*>(A + (size_t)srcs[i] * K + k + 8 * spiece) : zero8;
+            __syncthreads();                         // the step before has read its rows
+#pragma unroll
+            for (int i = 0; i < MT; ++i)
+                if (i < run) *reinterpret_cast<moe_bf16x8_t*>(xs + (srow + 16 * i) * MOE_LDS_STRIDE + 8 * spiece) = stage[i];
+            __syncthreads();
+            if (cols) {
+#pragma unroll
+                for (int j = 0; j < 4; ++j)
+#pragma unroll
+                    for (int mt = 0; mt < MT; ++mt)
+                        if (mt < run) {
+                            const moe_bf16x8_t b = *reinterpret_cast<const moe_bf16x8_t*>(xs + (mt * 16 + r) * MOE_LDS_STRIDE + 32 * j + 8 * g);
+#pragma unroll
+                            for (int nt = 0; nt < NT; ++nt) acc[nt][mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[nt][j], b, acc[nt][mt], 0, 0, 0);
+                        }
+            }
+        }
+        if (cols) {
+#pragma unroll
+            for (int mt = 0; mt < MT; ++mt) {
+                if (mt >= run || !xok[mt]) continue;
+                const size_t row = (size_t)(t + mt) * MOE_TM + r;
+                if (GATED) {
+#pragma unroll
+                    for (int i = 0; i < 4; ++i) {
+                        const int col = n0 + 4 * g + i;
+                        if (col < N) {
+                            const float gt = acc[0][mt][i];
+                            C[row * N + col] = from_f32<TC>(gt / (1.0f + expf(-gt)) * acc[1][mt][i]);
+                        }
+                    }
+                } else {
+#pragma unroll
+                    for (int nt = 0; nt < NT; ++nt)
+#pragma unroll
+                        for (int i = 0; i < 4; ++i) {
+                            const int col = n0 + nt * 16 + 4 * g + i;
+                            if (col < N) C[row * N + col] = from_f32<TC>(acc[nt][mt][i]);
+                        }
+                }
+            }
+        }
+        t += run;
+    }
+}
+
 template <int MT>
 static int moe_gemm_mfma_launch(void* C, int c_dtype, const void* A, const void* W, const int* tile_expert, const int* sorted_pair,
                                 int gather, int gated, int max_tiles, int N, int K, hipStream_t st) {
@@ -334,7 +447,15 @@ static int moe_gemm_mfma_launch(void* C, int c_dtype, const void* A, const void*
     const int cols = gated ? 64 : 128;
     const dim3 grid((max_tiles + MT - 1) / MT, (N + cols - 1) / cols);
     SPY_REQUIRE(grid.y <= 65535, "spy_moe_gemm: too many columns");
-    if (gated) {
+    if (MT == 8) {
+        if (gated) {
+            SPY_DISPATCH(c_dtype, TC, (moe_gemm_mfma_lds_kernel<true, TC><<<grid, 256, 0, st>>>((TC*)C, (const bf16_t*)A, (const bf16_t*)W, tile_expert,
+                                                                                               sorted_pair, gather, max_tiles, N, K, ws)));
+        } else {
+            SPY_DISPATCH(c_dtype, TC, (moe_gemm_mfma_lds_kernel<false, TC><<<grid, 256, 0, st>>>((TC*)C, (const bf16_t*)A, (const bf16_t*)W, tile_expert,
+                                                                                                sorted_pair, gather, max_tiles, N, K, ws)));
+        }
+    } else if (gated) {
         SPY_DISPATCH(c_dtype, TC, (moe_gemm_mfma_kernel<MT, true, TC><<<grid, 256, 0, st>>>((TC*)C, (const bf16_t*)A, (const bf16_t*)W, tile_expert,
                                                                                            sorted_pair, gather, max_tiles, N, K, ws)));
     } else {

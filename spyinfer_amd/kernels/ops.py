@@ -1212,7 +1212,7 @@ def mlstm(x: torch.Tensor, q_off: int, k_off: int, v_off: int, g_off: int, gates
           dv: int) -> torch.Tensor:
     """The mLSTM recurrence over the step's tokens.  ``x``: rows of the fused projection with q (H heads of d) at column
     ``q_off``, k at ``k_off``, v (H heads of dv) at ``v_off`` and the output gate's rows at ``g_off``; ``gates [T, 2 H]``
-    float32: the raw products of the input and forget gates (their biases ``bi``, ``bf [H]``; both capped by
+    float32: the raw products of the input and forget gates, overwritten with the log gates (their biases ``bi``, ``bf [H]``; both capped by
     cap tanh(. / cap)); ``state [slots, mlstm_state_size(H, d, dv)]`` float32 holds S, n and the running maximum of every
     head, read at an entry's start and left at its end.  Returns [T, H dv]: each head's read-out over its root mean square, times
     ``norm_w``, times sigmoid(gate)."""
@@ -1267,7 +1267,7 @@ def delta_rule(qkv: torch.Tensor, beta_pre: torch.Tensor, dec_pre: torch.Tensor,
                H: int, G: int, d: int, dv: int) -> torch.Tensor:
     """The gated delta rule over the step's tokens.  ``qkv [T, 2 G d + H dv]``: q and k (G heads of d; made unit vectors
     here, q also times d^-1/2) and v (H heads of dv); ``beta_pre [T, H]`` and ``dec_pre [T, H d]`` float32: the raw products
-    behind beta = sigmoid(.) and the decay exp(-exp(a_log[h]) softplus(. + dt_bias)) per head and key channel; per head
+    (overwritten with what they turn into) behind beta = sigmoid(.) and the decay exp(-exp(a_log[h]) softplus(. + dt_bias)) per head and key channel; per head
     S = diag(decay) S, u = beta (v - S^T k), S += k u^T, o = S^T q with ``state[slot, h d dv ..]`` float32.  Returns
     [T, H dv]: o over its root mean square, times ``norm_w [dv]``, times sigmoid(``gate``) (rows of H dv values, a view
     into a wider product allowed)."""
@@ -1287,7 +1287,8 @@ def delta_rule(qkv: torch.Tensor, beta_pre: torch.Tensor, dec_pre: torch.Tensor,
     out = torch.empty((T, H * dv), dtype=qkv.dtype, device=qkv.device)
     if T:
         tmp = torch.empty((T, H * dv), dtype=torch.float32, device=qkv.device)      # the read-outs before the heads' norm
-        hip().call("spy_delta_rule", _ptr(out), _ptr(tmp), _ptr(state), ctypes.c_longlong(state.shape[1]), _ptr(qkv), _code(qkv, "qkv"), _ptr(beta_pre),
+        unit = torch.empty((T, 2 * G * d), dtype=torch.float32, device=qkv.device)  # q and k as unit vectors
+        hip().call("spy_delta_rule", _ptr(out), _ptr(tmp), _ptr(unit), _ptr(state), ctypes.c_longlong(state.shape[1]), _ptr(qkv), _code(qkv, "qkv"), _ptr(beta_pre),
                    _ptr(dec_pre), _ptr(a_log), _ptr(dt_bias), _code(a_log, "decay numbers"), ctypes.c_void_p(gate.data_ptr()), ctypes.c_longlong(gs),
                    _ptr(norm_w), ctypes.c_float(eps), _ptr(cu_q), _ptr(slot_ids), ctypes.c_int(state.shape[0]), ctypes.c_int(S), ctypes.c_int(T),
                    ctypes.c_int(H), ctypes.c_int(G), ctypes.c_int(d), ctypes.c_int(dv), _Hip.stream())
