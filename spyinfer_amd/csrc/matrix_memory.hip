@@ -54,13 +54,14 @@ __global__ void mlstm_gates_kernel(float* __restrict__ gates, const TW* __restri
 // dv).  gates [T, 2 H] float32: the log input and forget gates (mlstm_gates_kernel).  state [slots][H][d dv + NS (d + 1)]:
 // S (row dd, column j at dd dv + j), then for every slice of 64 columns its own copy of n and m (the slices' waves do
 // not wait for each other, so none may read what another has already moved on).
+#define MM_AHEAD 4          // tokens whose operands are in flight ahead of the one being worked on
 template <typename TA, typename TW, int DR>
 __global__ __launch_bounds__(MM_SLICE) void mlstm_kernel(
     float* __restrict__ o_out, float* __restrict__ state, const TA* __restrict__ x, long long xs, int q_off, int k_off, int v_off,
     const float* __restrict__ gates, const int* __restrict__ cu_q,
     const int* __restrict__ slot_ids, int num_slots, int H, int d, int dv, int NS) {
-    __shared__ __align__(16) float ks[DR], qs[DR];
-    constexpr int R = DR / MM_SLICE;
+    constexpr int R = (DR + MM_SLICE - 1) / MM_SLICE, LD = R * MM_SLICE;
+    __shared__ __align__(16) float ks[LD], qs[LD];
     const int s = blockIdx.x, h = blockIdx.y, c = blockIdx.z, lane = threadIdx.x;
     const int j = c * MM_SLICE + lane;
     const int slot = slot_ids[s];
@@ -69,6 +70,8 @@ __global__ __launch_bounds__(MM_SLICE) void mlstm_kernel(
     float* st = state + ((size_t)slot * H + h) * head_state;
     float* nm = st + (size_t)d * dv + (size_t)c * (d + 1);
     const bool col = j < dv;
+    // rows of S beyond d stay zero, and so do the staged k and q there: the loops below run over all DR rows without
+    // conditions (straight-line code, so that the LDS reads go out ahead of the arithmetic)
     float S[DR];
 #pragma unroll
     for (int dd = 0; dd < DR; ++dd) S[dd] = (col && dd < d) ? st[(size_t)dd * dv + j] : 0.f;
@@ -83,58 +86,60 @@ __global__ __launch_bounds__(MM_SLICE) void mlstm_kernel(
     float m = nm[d];
     const float qscale = 1.0f / sqrtf((float)d);
     const int t0 = cu_q[s], t1 = cu_q[s + 1];
-    float kc[R], qc[R], vc = 0.f, gic = 0.f, gfc = 0.f;
-    float kn[R], qn[R], vn = 0.f, gin = 0.f, gfn = 0.f;
-#define MLSTM_LOAD(K, Q, V, GI, GF, TT)                                                        \
-    {                                                                                          \
-        const TA* xr_ = x + (size_t)(TT) * xs;                                                 \
-        _Pragma("unroll") for (int i = 0; i < R; ++i) {                                        \
-            const int idx = lane + MM_SLICE * i;                                               \
-            K[i] = idx < d ? to_f32<TA>(xr_[k_off + (size_t)h * d + idx]) : 0.f;               \
-            Q[i] = idx < d ? to_f32<TA>(xr_[q_off + (size_t)h * d + idx]) * qscale : 0.f;      \
-        }                                                                                      \
-        V = col ? to_f32<TA>(xr_[v_off + (size_t)h * dv + j]) : 0.f;                           \
-        GI = gates[(size_t)(TT) * 2 * H + h];                                                  \
-        GF = gates[(size_t)(TT) * 2 * H + H + h];                                              \
+    float kr[MM_AHEAD][R], qr[MM_AHEAD][R], vr[MM_AHEAD], gir[MM_AHEAD], gfr[MM_AHEAD];
+#define MLSTM_LOAD(U, TT)                                                                        \
+    if ((TT) < t1) {                                                                             \
+        const TA* xr_ = x + (size_t)(TT) * xs;                                                   \
+        _Pragma("unroll") for (int i = 0; i < R; ++i) {                                          \
+            const int idx = lane + MM_SLICE * i;                                                 \
+            kr[U][i] = idx < d ? to_f32<TA>(xr_[k_off + (size_t)h * d + idx]) : 0.f;             \
+            qr[U][i] = idx < d ? to_f32<TA>(xr_[q_off + (size_t)h * d + idx]) * qscale : 0.f;    \
+        }                                                                                        \
+        vr[U] = col ? to_f32<TA>(xr_[v_off + (size_t)h * dv + j]) : 0.f;                         \
+        gir[U] = gates[(size_t)(TT) * 2 * H + h];                                                \
+        gfr[U] = gates[(size_t)(TT) * 2 * H + H + h];                                            \
     }
-    if (t0 < t1) MLSTM_LOAD(kc, qc, vc, gic, gfc, t0)
-    for (int t = t0; t < t1; ++t) {
-        if (t + 1 < t1) MLSTM_LOAD(kn, qn, vn, gin, gfn, t + 1)
 #pragma unroll
-        for (int i = 0; i < R; ++i) {
-            const int idx = lane + MM_SLICE * i;
-            if (idx < d) { ks[idx] = kc[i]; qs[idx] = qc[i]; }
-        }
-        const float ig = gic, fg = gfc;
-        const float m_new = fmaxf(fg + m, ig);
-        const float a = expf(fg + m - m_new), b = expf(ig - m_new);
-        m = m_new;
-        __syncthreads();
-        float acc = 0.f;
-        const float bv = b * vc;
+    for (int u = 0; u < MM_AHEAD; ++u) MLSTM_LOAD(u, t0 + u)
+    for (int tb = t0; tb < t1; tb += MM_AHEAD) {
 #pragma unroll
-        for (int dd = 0; dd < DR; dd += 4) {
-            if (dd < d) {
-                const float4 k4 = *reinterpret_cast<const float4*>(ks + dd), q4 = *reinterpret_cast<const float4*>(qs + dd);
-                S[dd] = fmaf(a, S[dd], k4.x * bv);         acc = fmaf(S[dd], q4.x, acc);
-                S[dd + 1] = fmaf(a, S[dd + 1], k4.y * bv); acc = fmaf(S[dd + 1], q4.y, acc);
-                S[dd + 2] = fmaf(a, S[dd + 2], k4.z * bv); acc = fmaf(S[dd + 2], q4.z, acc);
-                S[dd + 3] = fmaf(a, S[dd + 3], k4.w * bv); acc = fmaf(S[dd + 3], q4.w, acc);
+        for (int u = 0; u < MM_AHEAD; ++u) {
+            const int t = tb + u;
+            if (t < t1) {
+#pragma unroll
+                for (int i = 0; i < R; ++i) {
+                    const int idx = lane + MM_SLICE * i;
+                    if (idx < d) { ks[idx] = kr[u][i]; qs[idx] = qr[u][i]; }
+                }
+                const float ig = gir[u], fg = gfr[u];
+                const float m_new = fmaxf(fg + m, ig);
+                const float a = expf(fg + m - m_new), b = expf(ig - m_new);
+                m = m_new;
+                __syncthreads();
+                float acc = 0.f, acc2 = 0.f;
+                const float bv = b * vr[u];
+#pragma unroll
+                for (int dd = 0; dd < DR; dd += 4) {
+                    const float4 k4 = *reinterpret_cast<const float4*>(ks + dd), q4 = *reinterpret_cast<const float4*>(qs + dd);
+                    S[dd] = fmaf(a, S[dd], k4.x * bv);         acc = fmaf(S[dd], q4.x, acc);
+                    S[dd + 1] = fmaf(a, S[dd + 1], k4.y * bv); acc2 = fmaf(S[dd + 1], q4.y, acc2);
+                    S[dd + 2] = fmaf(a, S[dd + 2], k4.z * bv); acc = fmaf(S[dd + 2], q4.z, acc);
+                    S[dd + 3] = fmaf(a, S[dd + 3], k4.w * bv); acc2 = fmaf(S[dd + 3], q4.w, acc2);
+                }
+                acc += acc2;
+                float nq = 0.f;
+#pragma unroll
+                for (int i = 0; i < R; ++i) {
+                    n[i] = fmaf(a, n[i], b * kr[u][i]);
+                    nq = fmaf(n[i], qr[u][i], nq);
+                }
+                nq = wave_sum(nq);
+                const float den = fmaxf(fabsf(nq), expf(-m)) + 1e-6f;
+                if (col) o_out[((size_t)t * H + h) * dv + j] = acc / den;
+                __syncthreads();
+                MLSTM_LOAD(u, t + MM_AHEAD)
             }
         }
-        float nq = 0.f;
-#pragma unroll
-        for (int i = 0; i < R; ++i) {
-            n[i] = fmaf(a, n[i], b * kc[i]);
-            nq = fmaf(n[i], qc[i], nq);
-        }
-        nq = wave_sum(nq);
-        const float den = fmaxf(fabsf(nq), expf(-m)) + 1e-6f;
-        if (col) o_out[((size_t)t * H + h) * dv + j] = acc / den;
-        __syncthreads();
-#pragma unroll
-        for (int i = 0; i < R; ++i) { kc[i] = kn[i]; qc[i] = qn[i]; }
-        vc = vn; gic = gin; gfc = gfn;
     }
 #undef MLSTM_LOAD
 #pragma unroll
@@ -150,7 +155,8 @@ __global__ __launch_bounds__(MM_SLICE) void mlstm_kernel(
 
 #define MM_LAUNCH(KERNEL, ...)                                                              \
     do {                                                                                    \
-        if (d <= 64) KERNEL<TA, TW, 64><<<grid, MM_SLICE, 0, st>>>(__VA_ARGS__);            \
+        if (d <= 32) KERNEL<TA, TW, 32><<<grid, MM_SLICE, 0, st>>>(__VA_ARGS__);            \
+        else if (d <= 64) KERNEL<TA, TW, 64><<<grid, MM_SLICE, 0, st>>>(__VA_ARGS__);       \
         else if (d <= 128) KERNEL<TA, TW, 128><<<grid, MM_SLICE, 0, st>>>(__VA_ARGS__);     \
         else KERNEL<TA, TW, 256><<<grid, MM_SLICE, 0, st>>>(__VA_ARGS__);                   \
     } while (0)
@@ -295,8 +301,8 @@ __global__ __launch_bounds__(MM_SLICE) void delta_rule_kernel(
     float* __restrict__ o_out, float* __restrict__ state, long long state_stride, const TA* __restrict__ qkv, const float* __restrict__ qk,
     const float* __restrict__ beta_pre, const float* __restrict__ dec_pre, const int* __restrict__ cu_q,
     const int* __restrict__ slot_ids, int num_slots, int H, int G, int d, int dv) {
-    __shared__ __align__(16) float ks[DR], qs[DR], dec[DR];
-    constexpr int R = DR / MM_SLICE;
+    constexpr int R = (DR + MM_SLICE - 1) / MM_SLICE, LD = R * MM_SLICE;
+    __shared__ __align__(16) float ks[LD], qs[LD], dec[LD];
     const int s = blockIdx.x, h = blockIdx.y, c = blockIdx.z, lane = threadIdx.x;
     const int j = c * MM_SLICE + lane;
     const int slot = slot_ids[s];
@@ -304,6 +310,7 @@ __global__ __launch_bounds__(MM_SLICE) void delta_rule_kernel(
     const int g = h / (H / G);
     float* st = state + (size_t)slot * state_stride + (size_t)h * d * dv;
     const bool col = j < dv;
+    // (rows beyond d: S zero, staged k and q zero, decay one; the loops run over all DR rows without conditions)
     float S[DR];
 #pragma unroll
     for (int dd = 0; dd < DR; ++dd) S[dd] = (col && dd < d) ? st[(size_t)dd * dv + j] : 0.f;
@@ -316,63 +323,57 @@ __global__ __launch_bounds__(MM_SLICE) void delta_rule_kernel(
     }
     const int C = 2 * G * d + H * dv;
     const int t0 = cu_q[s], t1 = cu_q[s + 1];
-    float kc[R], qc[R], zc[R], vc = 0.f, bc = 0.f;
-    float kn[R], qn[R], zn[R], vn = 0.f, bn = 0.f;
-#define DELTA_LOAD(K, Q, Z, V, B, TT)                                                          \
-    {                                                                                          \
-        const TA* xr_ = qkv + (size_t)(TT) * C;                                                \
-        const float* qk_ = qk + (size_t)(TT) * 2 * G * d;                                      \
-        _Pragma("unroll") for (int i = 0; i < R; ++i) {                                        \
-            const int idx = lane + MM_SLICE * i;                                               \
-            Q[i] = idx < d ? qk_[(size_t)g * d + idx] : 0.f;                                   \
-            K[i] = idx < d ? qk_[(size_t)(G + g) * d + idx] : 0.f;                             \
-            Z[i] = idx < d ? dec_pre[((size_t)(TT) * H + h) * d + idx] : 1.f;                  \
-        }                                                                                      \
-        V = col ? to_f32<TA>(xr_[(size_t)2 * G * d + (size_t)h * dv + j]) : 0.f;               \
-        B = beta_pre[(size_t)(TT) * H + h];                                                    \
+    float kr[MM_AHEAD][R], qr[MM_AHEAD][R], zr[MM_AHEAD][R], vr[MM_AHEAD], br[MM_AHEAD];
+#define DELTA_LOAD(U, TT)                                                                        \
+    if ((TT) < t1) {                                                                             \
+        const float* qk_ = qk + (size_t)(TT) * 2 * G * d;                                        \
+        _Pragma("unroll") for (int i = 0; i < R; ++i) {                                          \
+            const int idx = lane + MM_SLICE * i;                                                 \
+            qr[U][i] = idx < d ? qk_[(size_t)g * d + idx] : 0.f;                                 \
+            kr[U][i] = idx < d ? qk_[(size_t)(G + g) * d + idx] : 0.f;                           \
+            zr[U][i] = idx < d ? dec_pre[((size_t)(TT) * H + h) * d + idx] : 1.f;                \
+        }                                                                                        \
+        vr[U] = col ? to_f32<TA>(qkv[(size_t)(TT) * C + (size_t)2 * G * d + (size_t)h * dv + j]) : 0.f; \
+        br[U] = beta_pre[(size_t)(TT) * H + h];                                                  \
     }
-    if (t0 < t1) DELTA_LOAD(kc, qc, zc, vc, bc, t0)
-    for (int t = t0; t < t1; ++t) {
-        if (t + 1 < t1) DELTA_LOAD(kn, qn, zn, vn, bn, t + 1)
 #pragma unroll
-        for (int i = 0; i < R; ++i) {
-            const int idx = lane + MM_SLICE * i;
-            if (idx < d) {
-                qs[idx] = qc[i];
-                ks[idx] = kc[i];
-                dec[idx] = zc[i];
+    for (int u = 0; u < MM_AHEAD; ++u) DELTA_LOAD(u, t0 + u)
+    for (int tb = t0; tb < t1; tb += MM_AHEAD) {
+#pragma unroll
+        for (int u = 0; u < MM_AHEAD; ++u) {
+            const int t = tb + u;
+            if (t < t1) {
+#pragma unroll
+                for (int i = 0; i < R; ++i) {
+                    const int idx = lane + MM_SLICE * i;
+                    if (idx < d) { qs[idx] = qr[u][i]; ks[idx] = kr[u][i]; dec[idx] = zr[u][i]; }
+                }
+                const float beta = br[u];
+                __syncthreads();
+                float r = 0.f, r2 = 0.f;
+#pragma unroll
+                for (int dd = 0; dd < DR; dd += 4) {
+                    const float4 k4 = *reinterpret_cast<const float4*>(ks + dd), g4 = *reinterpret_cast<const float4*>(dec + dd);
+                    S[dd] *= g4.x;     r = fmaf(S[dd], k4.x, r);
+                    S[dd + 1] *= g4.y; r2 = fmaf(S[dd + 1], k4.y, r2);
+                    S[dd + 2] *= g4.z; r = fmaf(S[dd + 2], k4.z, r);
+                    S[dd + 3] *= g4.w; r2 = fmaf(S[dd + 3], k4.w, r2);
+                }
+                const float uu = beta * (vr[u] - (r + r2));
+                float acc = 0.f, acc2 = 0.f;
+#pragma unroll
+                for (int dd = 0; dd < DR; dd += 4) {
+                    const float4 k4 = *reinterpret_cast<const float4*>(ks + dd), q4 = *reinterpret_cast<const float4*>(qs + dd);
+                    S[dd] = fmaf(k4.x, uu, S[dd]);         acc = fmaf(S[dd], q4.x, acc);
+                    S[dd + 1] = fmaf(k4.y, uu, S[dd + 1]); acc2 = fmaf(S[dd + 1], q4.y, acc2);
+                    S[dd + 2] = fmaf(k4.z, uu, S[dd + 2]); acc = fmaf(S[dd + 2], q4.z, acc);
+                    S[dd + 3] = fmaf(k4.w, uu, S[dd + 3]); acc2 = fmaf(S[dd + 3], q4.w, acc2);
+                }
+                if (col) o_out[((size_t)t * H + h) * dv + j] = acc + acc2;
+                __syncthreads();
+                DELTA_LOAD(u, t + MM_AHEAD)
             }
         }
-        const float beta = bc;
-        __syncthreads();
-        float r = 0.f;
-#pragma unroll
-        for (int dd = 0; dd < DR; dd += 4) {
-            if (dd < d) {
-                const float4 k4 = *reinterpret_cast<const float4*>(ks + dd), g4 = *reinterpret_cast<const float4*>(dec + dd);
-                S[dd] *= g4.x;     r = fmaf(S[dd], k4.x, r);
-                S[dd + 1] *= g4.y; r = fmaf(S[dd + 1], k4.y, r);
-                S[dd + 2] *= g4.z; r = fmaf(S[dd + 2], k4.z, r);
-                S[dd + 3] *= g4.w; r = fmaf(S[dd + 3], k4.w, r);
-            }
-        }
-        const float u = beta * (vc - r);
-        float acc = 0.f;
-#pragma unroll
-        for (int dd = 0; dd < DR; dd += 4) {
-            if (dd < d) {
-                const float4 k4 = *reinterpret_cast<const float4*>(ks + dd), q4 = *reinterpret_cast<const float4*>(qs + dd);
-                S[dd] = fmaf(k4.x, u, S[dd]);         acc = fmaf(S[dd], q4.x, acc);
-                S[dd + 1] = fmaf(k4.y, u, S[dd + 1]); acc = fmaf(S[dd + 1], q4.y, acc);
-                S[dd + 2] = fmaf(k4.z, u, S[dd + 2]); acc = fmaf(S[dd + 2], q4.z, acc);
-                S[dd + 3] = fmaf(k4.w, u, S[dd + 3]); acc = fmaf(S[dd + 3], q4.w, acc);
-            }
-        }
-        if (col) o_out[((size_t)t * H + h) * dv + j] = acc;
-        __syncthreads();
-#pragma unroll
-        for (int i = 0; i < R; ++i) { kc[i] = kn[i]; qc[i] = qn[i]; zc[i] = zn[i]; }
-        vc = vn; bc = bn;
     }
 #undef DELTA_LOAD
 #pragma unroll
