@@ -1,7 +1,8 @@
 // Recurrent mixers whose state is a matrix per head, S [d, dv] in float32 in the request's slot: a write k v^T per
-// token, a read-out S^T q.  One wave per (entry, head, slice of 64 value channels); lane j owns one column of S (the d
-// values that belong to its value channel) in registers and walks the entry's tokens; the token's key and query go
-// through LDS, and the next token's operands are asked for before this token's arithmetic.  The read-outs leave as
+// token, a read-out S^T q.  One wave per (entry, head, slice of 16 value channels): four neighbouring lanes share a
+// column of S, each with a quarter of its d rows in registers, and add their parts of a sum with two DPP exchanges
+// inside the quad (no LDS, no barrier); the wave walks the entry's tokens; the token's key and query go through LDS,
+// and the operands of the next four tokens are in flight ahead of this token's arithmetic.  The read-outs leave as
 // float32; a second kernel norms every head over all its slices, applies weight and gate and rounds once.
 // Everything behind the projections is float32.
 //
@@ -16,7 +17,15 @@
 __device__ __forceinline__ float mm_sigmoid(float x) { return 1.0f / (1.0f + expf(-x)); }
 __device__ __forceinline__ float mm_logsigmoid(float x) { return fminf(x, 0.f) - log1pf(expf(-fabsf(x))); }
 
-#define MM_SLICE 64
+#define MM_SLICE 64          // lanes of a block (one wave)
+#define MM_COLS 16           // value channels of a wave: four lanes a column
+
+// sum over the four lanes of a quad, in every one of them
+__device__ __forceinline__ float quad_sum(float x) {
+    x += __int_as_float(__builtin_amdgcn_mov_dpp(__float_as_int(x), 0xB1, 0xF, 0xF, true));      // lanes 1 0 3 2
+    x += __int_as_float(__builtin_amdgcn_mov_dpp(__float_as_int(x), 0x4E, 0xF, 0xF, true));      // lanes 2 3 0 1
+    return x;
+}
 
 // out[t, h, j] = o[t, h, j] / sqrt(mean_j(o[t, h, :]^2) + eps) * w[(per_head ? h dv : 0) + j] * sigmoid(gate[t, h dv + j]);
 // one block per (token, head)
@@ -52,7 +61,7 @@ __global__ void mlstm_gates_kernel(float* __restrict__ gates, const TW* __restri
 
 // x: rows of the fused projection, xs values apart; q at column q_off (H heads of d), k at k_off, v at v_off (H heads of
 // dv).  gates [T, 2 H] float32: the log input and forget gates (mlstm_gates_kernel).  state [slots][H][d dv + NS (d + 1)]:
-// S (row dd, column j at dd dv + j), then for every slice of 64 columns its own copy of n and m (the slices' waves do
+// S (row dd, column j at dd dv + j), then for every slice of 16 columns its own copy of n and m (the slices' waves do
 // not wait for each other, so none may read what another has already moved on).
 #define MM_AHEAD 4          // tokens whose operands are in flight ahead of the one being worked on
 template <typename TA, typename TW, int DR>
@@ -60,28 +69,29 @@ __global__ __launch_bounds__(MM_SLICE) void mlstm_kernel(
     float* __restrict__ o_out, float* __restrict__ state, const TA* __restrict__ x, long long xs, int q_off, int k_off, int v_off,
     const float* __restrict__ gates, const int* __restrict__ cu_q,
     const int* __restrict__ slot_ids, int num_slots, int H, int d, int dv, int NS) {
-    constexpr int R = (DR + MM_SLICE - 1) / MM_SLICE, LD = R * MM_SLICE;
+    constexpr int R = (DR + MM_SLICE - 1) / MM_SLICE, LD = R * MM_SLICE, DQ = DR / 4;
     __shared__ __align__(16) float ks[LD], qs[LD];
     const int s = blockIdx.x, h = blockIdx.y, c = blockIdx.z, lane = threadIdx.x;
-    const int j = c * MM_SLICE + lane;
+    const int part = lane & 3, j = c * MM_COLS + (lane >> 2);
+    const int row0 = part * DQ;                       // this lane's rows of S: row0 .. row0 + DQ - 1
     const int slot = slot_ids[s];
     if (slot < 0 || slot >= num_slots) return;
     const size_t head_state = (size_t)d * dv + (size_t)NS * (d + 1);
     float* st = state + ((size_t)slot * H + h) * head_state;
     float* nm = st + (size_t)d * dv + (size_t)c * (d + 1);
     const bool col = j < dv;
-    // rows of S beyond d stay zero, and so do the staged k and q there: the loops below run over all DR rows without
-    // conditions (straight-line code, so that the LDS reads go out ahead of the arithmetic)
-    float S[DR];
+    // rows of S beyond d stay zero, and so do the staged k and q there: the loops below run over all of a lane's rows
+    // without conditions (straight-line code, so that the LDS reads go out ahead of the arithmetic)
+    float S[DQ], n[DQ];
 #pragma unroll
-    for (int dd = 0; dd < DR; ++dd) S[dd] = (col && dd < d) ? st[(size_t)dd * dv + j] : 0.f;
-    float n[R];
+    for (int i = 0; i < DQ; ++i) {
+        S[i] = (col && row0 + i < d) ? st[(size_t)(row0 + i) * dv + j] : 0.f;
+        n[i] = row0 + i < d ? nm[row0 + i] : 0.f;
+    }
 #pragma unroll
     for (int i = 0; i < R; ++i) {
-        const int idx = lane + MM_SLICE * i;
-        n[i] = idx < d ? nm[idx] : 0.f;
-        ks[idx] = 0.f;
-        qs[idx] = 0.f;
+        ks[lane + MM_SLICE * i] = 0.f;
+        qs[lane + MM_SLICE * i] = 0.f;
     }
     float m = nm[d];
     const float qscale = 1.0f / sqrtf((float)d);
@@ -116,26 +126,24 @@ __global__ __launch_bounds__(MM_SLICE) void mlstm_kernel(
                 const float a = expf(fg + m - m_new), b = expf(ig - m_new);
                 m = m_new;
                 __syncthreads();
-                float acc = 0.f, acc2 = 0.f;
+                float acc = 0.f, nq = 0.f;
                 const float bv = b * vr[u];
 #pragma unroll
-                for (int dd = 0; dd < DR; dd += 4) {
-                    const float4 k4 = *reinterpret_cast<const float4*>(ks + dd), q4 = *reinterpret_cast<const float4*>(qs + dd);
-                    S[dd] = fmaf(a, S[dd], k4.x * bv);         acc = fmaf(S[dd], q4.x, acc);
-                    S[dd + 1] = fmaf(a, S[dd + 1], k4.y * bv); acc2 = fmaf(S[dd + 1], q4.y, acc2);
-                    S[dd + 2] = fmaf(a, S[dd + 2], k4.z * bv); acc = fmaf(S[dd + 2], q4.z, acc);
-                    S[dd + 3] = fmaf(a, S[dd + 3], k4.w * bv); acc2 = fmaf(S[dd + 3], q4.w, acc2);
+                for (int i = 0; i < DQ; i += 4) {
+                    const float4 k4 = *reinterpret_cast<const float4*>(ks + row0 + i), q4 = *reinterpret_cast<const float4*>(qs + row0 + i);
+                    S[i] = fmaf(a, S[i], k4.x * bv);         acc = fmaf(S[i], q4.x, acc);
+                    S[i + 1] = fmaf(a, S[i + 1], k4.y * bv); acc = fmaf(S[i + 1], q4.y, acc);
+                    S[i + 2] = fmaf(a, S[i + 2], k4.z * bv); acc = fmaf(S[i + 2], q4.z, acc);
+                    S[i + 3] = fmaf(a, S[i + 3], k4.w * bv); acc = fmaf(S[i + 3], q4.w, acc);
+                    n[i] = fmaf(a, n[i], b * k4.x);         nq = fmaf(n[i], q4.x, nq);
+                    n[i + 1] = fmaf(a, n[i + 1], b * k4.y); nq = fmaf(n[i + 1], q4.y, nq);
+                    n[i + 2] = fmaf(a, n[i + 2], b * k4.z); nq = fmaf(n[i + 2], q4.z, nq);
+                    n[i + 3] = fmaf(a, n[i + 3], b * k4.w); nq = fmaf(n[i + 3], q4.w, nq);
                 }
-                acc += acc2;
-                float nq = 0.f;
-#pragma unroll
-                for (int i = 0; i < R; ++i) {
-                    n[i] = fmaf(a, n[i], b * kr[u][i]);
-                    nq = fmaf(n[i], qr[u][i], nq);
-                }
-                nq = wave_sum(nq);
+                acc = quad_sum(acc);
+                nq = quad_sum(nq);
                 const float den = fmaxf(fabsf(nq), expf(-m)) + 1e-6f;
-                if (col) o_out[((size_t)t * H + h) * dv + j] = acc / den;
+                if (col && part == 0) o_out[((size_t)t * H + h) * dv + j] = acc / den;
                 __syncthreads();
                 MLSTM_LOAD(u, t + MM_AHEAD)
             }
@@ -143,12 +151,9 @@ __global__ __launch_bounds__(MM_SLICE) void mlstm_kernel(
     }
 #undef MLSTM_LOAD
 #pragma unroll
-    for (int dd = 0; dd < DR; ++dd)
-        if (col && dd < d) st[(size_t)dd * dv + j] = S[dd];
-#pragma unroll
-    for (int i = 0; i < R; ++i) {
-        const int idx = lane + MM_SLICE * i;
-        if (idx < d) nm[idx] = n[i];
+    for (int i = 0; i < DQ; ++i) {
+        if (col && row0 + i < d) st[(size_t)(row0 + i) * dv + j] = S[i];
+        if (lane < 4 && row0 + i < d) nm[row0 + i] = n[i];
     }
     if (lane == 0) nm[d] = m;
 }
@@ -167,7 +172,7 @@ extern "C" int spy_mlstm(void* out, float* o_tmp, float* state, const void* x, l
     SPY_REQUIRE(S > 0 && T > 0 && H > 0 && d > 0 && dv > 0 && num_slots > 0 && o_tmp, "spy_mlstm: empty operand");
     SPY_REQUIRE(d <= 256 && dv <= 1024 && H <= 65535, "spy_mlstm: heads of %d x %d (key size up to 256, value size up to 1024)", d, dv);
     SPY_REQUIRE(cap > 0.f, "spy_mlstm: the gates' cap must be positive");
-    const int NS = (dv + MM_SLICE - 1) / MM_SLICE;
+    const int NS = (dv + MM_COLS - 1) / MM_COLS;
     const dim3 grid(S, H, NS);
     {
         const size_t total = (size_t)T * 2 * H;
@@ -301,25 +306,25 @@ __global__ __launch_bounds__(MM_SLICE) void delta_rule_kernel(
     float* __restrict__ o_out, float* __restrict__ state, long long state_stride, const TA* __restrict__ qkv, const float* __restrict__ qk,
     const float* __restrict__ beta_pre, const float* __restrict__ dec_pre, const int* __restrict__ cu_q,
     const int* __restrict__ slot_ids, int num_slots, int H, int G, int d, int dv) {
-    constexpr int R = (DR + MM_SLICE - 1) / MM_SLICE, LD = R * MM_SLICE;
+    constexpr int R = (DR + MM_SLICE - 1) / MM_SLICE, LD = R * MM_SLICE, DQ = DR / 4;
     __shared__ __align__(16) float ks[LD], qs[LD], dec[LD];
     const int s = blockIdx.x, h = blockIdx.y, c = blockIdx.z, lane = threadIdx.x;
-    const int j = c * MM_SLICE + lane;
+    const int part = lane & 3, j = c * MM_COLS + (lane >> 2);
+    const int row0 = part * DQ;
     const int slot = slot_ids[s];
     if (slot < 0 || slot >= num_slots) return;
     const int g = h / (H / G);
     float* st = state + (size_t)slot * state_stride + (size_t)h * d * dv;
     const bool col = j < dv;
-    // (rows beyond d: S zero, staged k and q zero, decay one; the loops run over all DR rows without conditions)
-    float S[DR];
+    // (rows beyond d: S zero, staged k and q zero, decay one; the loops run over all of a lane's rows without conditions)
+    float S[DQ];
 #pragma unroll
-    for (int dd = 0; dd < DR; ++dd) S[dd] = (col && dd < d) ? st[(size_t)dd * dv + j] : 0.f;
+    for (int i = 0; i < DQ; ++i) S[i] = (col && row0 + i < d) ? st[(size_t)(row0 + i) * dv + j] : 0.f;
 #pragma unroll
     for (int i = 0; i < R; ++i) {
-        const int idx = lane + MM_SLICE * i;
-        ks[idx] = 0.f;
-        qs[idx] = 0.f;
-        dec[idx] = 1.f;
+        ks[lane + MM_SLICE * i] = 0.f;
+        qs[lane + MM_SLICE * i] = 0.f;
+        dec[lane + MM_SLICE * i] = 1.f;
     }
     const int C = 2 * G * d + H * dv;
     const int t0 = cu_q[s], t1 = cu_q[s + 1];
@@ -350,26 +355,27 @@ __global__ __launch_bounds__(MM_SLICE) void delta_rule_kernel(
                 }
                 const float beta = br[u];
                 __syncthreads();
-                float r = 0.f, r2 = 0.f;
+                float r = 0.f;
 #pragma unroll
-                for (int dd = 0; dd < DR; dd += 4) {
-                    const float4 k4 = *reinterpret_cast<const float4*>(ks + dd), g4 = *reinterpret_cast<const float4*>(dec + dd);
-                    S[dd] *= g4.x;     r = fmaf(S[dd], k4.x, r);
-                    S[dd + 1] *= g4.y; r2 = fmaf(S[dd + 1], k4.y, r2);
-                    S[dd + 2] *= g4.z; r = fmaf(S[dd + 2], k4.z, r);
-                    S[dd + 3] *= g4.w; r2 = fmaf(S[dd + 3], k4.w, r2);
+                for (int i = 0; i < DQ; i += 4) {
+                    const float4 k4 = *reinterpret_cast<const float4*>(ks + row0 + i), g4 = *reinterpret_cast<const float4*>(dec + row0 + i);
+                    S[i] *= g4.x;     r = fmaf(S[i], k4.x, r);
+                    S[i + 1] *= g4.y; r = fmaf(S[i + 1], k4.y, r);
+                    S[i + 2] *= g4.z; r = fmaf(S[i + 2], k4.z, r);
+                    S[i + 3] *= g4.w; r = fmaf(S[i + 3], k4.w, r);
                 }
-                const float uu = beta * (vr[u] - (r + r2));
-                float acc = 0.f, acc2 = 0.f;
+                const float uu = beta * (vr[u] - quad_sum(r));
+                float acc = 0.f;
 #pragma unroll
-                for (int dd = 0; dd < DR; dd += 4) {
-                    const float4 k4 = *reinterpret_cast<const float4*>(ks + dd), q4 = *reinterpret_cast<const float4*>(qs + dd);
-                    S[dd] = fmaf(k4.x, uu, S[dd]);         acc = fmaf(S[dd], q4.x, acc);
-                    S[dd + 1] = fmaf(k4.y, uu, S[dd + 1]); acc2 = fmaf(S[dd + 1], q4.y, acc2);
-                    S[dd + 2] = fmaf(k4.z, uu, S[dd + 2]); acc = fmaf(S[dd + 2], q4.z, acc);
-                    S[dd + 3] = fmaf(k4.w, uu, S[dd + 3]); acc2 = fmaf(S[dd + 3], q4.w, acc2);
+                for (int i = 0; i < DQ; i += 4) {
+                    const float4 k4 = *reinterpret_cast<const float4*>(ks + row0 + i), q4 = *reinterpret_cast<const float4*>(qs + row0 + i);
+                    S[i] = fmaf(k4.x, uu, S[i]);         acc = fmaf(S[i], q4.x, acc);
+                    S[i + 1] = fmaf(k4.y, uu, S[i + 1]); acc = fmaf(S[i + 1], q4.y, acc);
+                    S[i + 2] = fmaf(k4.z, uu, S[i + 2]); acc = fmaf(S[i + 2], q4.z, acc);
+                    S[i + 3] = fmaf(k4.w, uu, S[i + 3]); acc = fmaf(S[i + 3], q4.w, acc);
                 }
-                if (col) o_out[((size_t)t * H + h) * dv + j] = acc + acc2;
+                acc = quad_sum(acc);
+                if (col && part == 0) o_out[((size_t)t * H + h) * dv + j] = acc;
                 __syncthreads();
                 DELTA_LOAD(u, t + MM_AHEAD)
             }
@@ -377,8 +383,8 @@ __global__ __launch_bounds__(MM_SLICE) void delta_rule_kernel(
     }
 #undef DELTA_LOAD
 #pragma unroll
-    for (int dd = 0; dd < DR; ++dd)
-        if (col && dd < d) st[(size_t)dd * dv + j] = S[dd];
+    for (int i = 0; i < DQ; ++i)
+        if (col && row0 + i < d) st[(size_t)(row0 + i) * dv + j] = S[i];
 }
 
 extern "C" int spy_delta_rule(void* out, float* o_tmp, float* qk_tmp, float* state, long long state_stride, const void* qkv, int dtype,
@@ -393,7 +399,7 @@ extern "C" int spy_delta_rule(void* out, float* o_tmp, float* qk_tmp, float* sta
     SPY_DISPATCH(dtype, TA, SPY_DISPATCH(w_dtype, TW, (delta_prepare_kernel<TA, TW><<<pgrid, 64, 0, st>>>(
         qk_tmp, (const TA*)qkv, beta_pre, dec_pre, (const TW*)a_log, (const TW*)dt_bias, H, G, d, dv))));
     SPY_CHECK_LAUNCH("spy_delta_rule (unit vectors and decays)");
-    const dim3 grid(S, H, (dv + MM_SLICE - 1) / MM_SLICE);
+    const dim3 grid(S, H, (dv + MM_COLS - 1) / MM_COLS);
     SPY_DISPATCH(dtype, TA, SPY_DISPATCH(w_dtype, TW, MM_LAUNCH(delta_rule_kernel, o_tmp, state, state_stride, (const TA*)qkv, qk_tmp, beta_pre,
         dec_pre, cu_q, slot_ids, num_slots, H, G, d, dv)));
     SPY_CHECK_LAUNCH("spy_delta_rule");

@@ -1192,7 +1192,7 @@ def sigmoid_gate(y: torch.Tensor, gate: torch.Tensor) -> torch.Tensor:
 # --------------------------------------------------------------------------
 # Recurrent mixers with a matrix state per head
 MATRIX_MEMORY_MAX_DIM, MATRIX_MEMORY_MAX_VDIM = 256, 1024
-MATRIX_MEMORY_SLICE = 64          # value channels that one wave of the recurrences owns
+MATRIX_MEMORY_SLICE = 16          # value channels that one wave of the recurrences owns (four lanes a channel)
 
 
 def mlstm_state_size(H: int, d: int, dv: int) -> int:
