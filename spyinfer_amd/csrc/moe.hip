@@ -382,23 +382,31 @@ __global__ __launch_bounds__(256) void moe_gemm_mfma_lds_kernel(TC* __restrict__
         for (int nt = 0; nt < NT; ++nt)
 #pragma unroll
             for (int mt = 0; mt < MT; ++mt) acc[nt][mt] = moe_f32x4_t{0.f, 0.f, 0.f, 0.f};
+        // the operands of a step are asked for one step ahead: W fragments into registers, the rows of A into registers
+        // on their way to LDS, both in flight while the matrix cores work on the step before
+        moe_bf16x8_t a[NT][4], stage[MT];
+#define MOE_ASK(KK)                                                                                                            \
+        {                                                                                                                      \
+            _Pragma("unroll") for (int j = 0; j < 4; ++j)                                                                      \
+                _Pragma("unroll") for (int nt = 0; nt < NT; ++nt)                                                              \
+                    a[nt][j] = (cols && (KK) + 32 * j + 8 * g < K) ? *reinterpret_cast<const moe_bf16x8_t*>(wrow[nt] + (KK) + 32 * j) : zero8; \
+            const bool kin_ = (KK) + 8 * spiece < K;                                                                           \
+            _Pragma("unroll") for (int i = 0; i < MT; ++i)                                                                     \
+                stage[i] = (i < run && srcs[i] >= 0 && kin_) ? *reinterpret_cast<const moe_bf16x8_t*>(A + (size_t)srcs[i] * K + (KK) + 8 * spiece) : zero8; \
+        }
+        MOE_ASK(0)
         for (int k = 0; k < K; k += 128) {
-            moe_bf16x8_t a[NT][4];
+            moe_bf16x8_t ac[NT][4];
 #pragma unroll
             for (int j = 0; j < 4; ++j)
 #pragma unroll
-                for (int nt = 0; nt < NT; ++nt)
-                    a[nt][j] = (cols && k + 32 * j + 8 * g < K) ? *reinterpret_cast<const moe_bf16x8_t*>(wrow[nt] + k + 32 * j) : zero8;
-            moe_bf16x8_t stage[MT];
-            const bool kin = k + 8 * spiece < K;
-#pragma unroll
-            for (int i = 0; i < MT; ++i)
-                stage[i] = (i < run && srcs[i] >= 0 && kin) ? *reinterpret_cast<const moe_bf16x8_t*>(A + (size_t)srcs[i] * K + k + 8 * spiece) : zero8;
+                for (int nt = 0; nt < NT; ++nt) ac[nt][j] = a[nt][j];
             __syncthreads();                         // the step before has read its rows
 #pragma unroll
             for (int i = 0; i < MT; ++i)
                 if (i < run) *reinterpret_cast<moe_bf16x8_t*>(xs + (srow + 16 * i) * MOE_LDS_STRIDE + 8 * spiece) = stage[i];
             __syncthreads();
+            if (k + 128 < K) MOE_ASK(k + 128)
             if (cols) {
 #pragma unroll
                 for (int j = 0; j < 4; ++j)
@@ -407,10 +415,11 @@ __global__ __launch_bounds__(256) void moe_gemm_mfma_lds_kernel(TC* __restrict__
                         if (mt < run) {
                             const moe_bf16x8_t b = *reinterpret_cast<const moe_bf16x8_t*>(xs + (mt * 16 + r) * MOE_LDS_STRIDE + 32 * j + 8 * g);
 #pragma unroll
-                            for (int nt = 0; nt < NT; ++nt) acc[nt][mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[nt][j], b, acc[nt][mt], 0, 0, 0);
+                            for (int nt = 0; nt < NT; ++nt) acc[nt][mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ac[nt][j], b, acc[nt][mt], 0, 0, 0);
                         }
             }
         }
+#undef MOE_ASK
         if (cols) {
 #pragma unroll
             for (int mt = 0; mt < MT; ++mt) {

@@ -217,7 +217,8 @@ def test_router_chooses_among_the_best_groups(E, top, groups, keep):
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
-@pytest.mark.parametrize("T,K,F,E,top", [(1, 48, 24, 8, 3), (37, 64, 40, 6, 2), (300, 128, 96, 12, 4), (5, 40, 8, 4, 4), (64, 256, 128, 130, 5)])
+@pytest.mark.parametrize("T,K,F,E,top", [(1, 48, 24, 8, 3), (37, 64, 40, 6, 2), (300, 128, 96, 12, 4), (5, 40, 8, 4, 4), (64, 256, 128, 130, 5),
+                                         (200, 1288, 72, 4, 2), (6, 1288, 48, 8, 2)])      # (many steps of K, the last one in part)
 def test_experts_over_sorted_pairs(dtype, T, K, F, E, top):
     from spyinfer_amd.kernels import ops
     dev = require_gpu()
