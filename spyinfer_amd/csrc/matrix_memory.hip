@@ -20,6 +20,15 @@ __device__ __forceinline__ float mm_logsigmoid(float x) { return fminf(x, 0.f) -
 #define MM_SLICE 64          // lanes of a block (one wave)
 #define MM_COLS 16           // value channels of a wave: four lanes a column
 
+// Between a wave's LDS writes and its own LDS reads: a block here is ONE wave, whose LDS operations run in program order,
+// so no barrier is needed, and none is wanted: a barrier would also wait for the global loads that are in flight for
+// the tokens ahead.  What is needed is that the compiler keeps the order.
+__device__ __forceinline__ void mm_wave_order() {
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+}
+
 // sum over the four lanes of a quad, in every one of them
 __device__ __forceinline__ float quad_sum(float x) {
     x += __int_as_float(__builtin_amdgcn_mov_dpp(__float_as_int(x), 0xB1, 0xF, 0xF, true));      // lanes 1 0 3 2
@@ -125,26 +134,26 @@ __global__ __launch_bounds__(MM_SLICE) void mlstm_kernel(
                 const float m_new = fmaxf(fg + m, ig);
                 const float a = expf(fg + m - m_new), b = expf(ig - m_new);
                 m = m_new;
-                __syncthreads();
-                float acc = 0.f, nq = 0.f;
+                mm_wave_order();
+                float acc = 0.f, acc2 = 0.f, nq = 0.f, nq2 = 0.f;
                 const float bv = b * vr[u];
 #pragma unroll
                 for (int i = 0; i < DQ; i += 4) {
                     const float4 k4 = *reinterpret_cast<const float4*>(ks + row0 + i), q4 = *reinterpret_cast<const float4*>(qs + row0 + i);
                     S[i] = fmaf(a, S[i], k4.x * bv);         acc = fmaf(S[i], q4.x, acc);
-                    S[i + 1] = fmaf(a, S[i + 1], k4.y * bv); acc = fmaf(S[i + 1], q4.y, acc);
+                    S[i + 1] = fmaf(a, S[i + 1], k4.y * bv); acc2 = fmaf(S[i + 1], q4.y, acc2);
                     S[i + 2] = fmaf(a, S[i + 2], k4.z * bv); acc = fmaf(S[i + 2], q4.z, acc);
-                    S[i + 3] = fmaf(a, S[i + 3], k4.w * bv); acc = fmaf(S[i + 3], q4.w, acc);
+                    S[i + 3] = fmaf(a, S[i + 3], k4.w * bv); acc2 = fmaf(S[i + 3], q4.w, acc2);
                     n[i] = fmaf(a, n[i], b * k4.x);         nq = fmaf(n[i], q4.x, nq);
-                    n[i + 1] = fmaf(a, n[i + 1], b * k4.y); nq = fmaf(n[i + 1], q4.y, nq);
+                    n[i + 1] = fmaf(a, n[i + 1], b * k4.y); nq2 = fmaf(n[i + 1], q4.y, nq2);
                     n[i + 2] = fmaf(a, n[i + 2], b * k4.z); nq = fmaf(n[i + 2], q4.z, nq);
-                    n[i + 3] = fmaf(a, n[i + 3], b * k4.w); nq = fmaf(n[i + 3], q4.w, nq);
+                    n[i + 3] = fmaf(a, n[i + 3], b * k4.w); nq2 = fmaf(n[i + 3], q4.w, nq2);
                 }
-                acc = quad_sum(acc);
-                nq = quad_sum(nq);
+                acc = quad_sum(acc + acc2);
+                nq = quad_sum(nq + nq2);
                 const float den = fmaxf(fabsf(nq), expf(-m)) + 1e-6f;
                 if (col && part == 0) o_out[((size_t)t * H + h) * dv + j] = acc / den;
-                __syncthreads();
+                mm_wave_order();
                 MLSTM_LOAD(u, t + MM_AHEAD)
             }
         }
@@ -354,29 +363,29 @@ __global__ __launch_bounds__(MM_SLICE) void delta_rule_kernel(
                     if (idx < d) { qs[idx] = qr[u][i]; ks[idx] = kr[u][i]; dec[idx] = zr[u][i]; }
                 }
                 const float beta = br[u];
-                __syncthreads();
-                float r = 0.f;
+                mm_wave_order();
+                float r = 0.f, r2 = 0.f;
 #pragma unroll
                 for (int i = 0; i < DQ; i += 4) {
                     const float4 k4 = *reinterpret_cast<const float4*>(ks + row0 + i), g4 = *reinterpret_cast<const float4*>(dec + row0 + i);
                     S[i] *= g4.x;     r = fmaf(S[i], k4.x, r);
-                    S[i + 1] *= g4.y; r = fmaf(S[i + 1], k4.y, r);
+                    S[i + 1] *= g4.y; r2 = fmaf(S[i + 1], k4.y, r2);
                     S[i + 2] *= g4.z; r = fmaf(S[i + 2], k4.z, r);
-                    S[i + 3] *= g4.w; r = fmaf(S[i + 3], k4.w, r);
+                    S[i + 3] *= g4.w; r2 = fmaf(S[i + 3], k4.w, r2);
                 }
-                const float uu = beta * (vr[u] - quad_sum(r));
-                float acc = 0.f;
+                const float uu = beta * (vr[u] - quad_sum(r + r2));
+                float acc = 0.f, acc2 = 0.f;
 #pragma unroll
                 for (int i = 0; i < DQ; i += 4) {
                     const float4 k4 = *reinterpret_cast<const float4*>(ks + row0 + i), q4 = *reinterpret_cast<const float4*>(qs + row0 + i);
                     S[i] = fmaf(k4.x, uu, S[i]);         acc = fmaf(S[i], q4.x, acc);
-                    S[i + 1] = fmaf(k4.y, uu, S[i + 1]); acc = fmaf(S[i + 1], q4.y, acc);
+                    S[i + 1] = fmaf(k4.y, uu, S[i + 1]); acc2 = fmaf(S[i + 1], q4.y, acc2);
                     S[i + 2] = fmaf(k4.z, uu, S[i + 2]); acc = fmaf(S[i + 2], q4.z, acc);
-                    S[i + 3] = fmaf(k4.w, uu, S[i + 3]); acc = fmaf(S[i + 3], q4.w, acc);
+                    S[i + 3] = fmaf(k4.w, uu, S[i + 3]); acc2 = fmaf(S[i + 3], q4.w, acc2);
                 }
-                acc = quad_sum(acc);
+                acc = quad_sum(acc + acc2);
                 if (col && part == 0) o_out[((size_t)t * H + h) * dv + j] = acc;
-                __syncthreads();
+                mm_wave_order();
                 DELTA_LOAD(u, t + MM_AHEAD)
             }
         }
