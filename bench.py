@@ -85,7 +85,7 @@ def sodedra_shape(width: int, layers: int, vocab: int, window: int = 1024) -> di
     for i in range(layers):
         kind = i % 4
         if kind == 0:
-            out.append(dict(type="mlstm", mixer=dict(heads=max(1, heads // 2), dim=128, vdim=256, gate_cap=15.0), mlp=dense))
+            out.append(dict(type="mlstm", mixer=dict(heads=max(1, heads // 2), dim=128, vdim=256, gate_cap=16.0), mlp=dense))
         elif kind == 1:
             out.append(dict(type="attention", mixer=dict(att), mlp=moe))
         elif kind == 2:

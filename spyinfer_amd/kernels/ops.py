@@ -341,15 +341,16 @@ def linear_few(x: torch.Tensor, w: torch.Tensor, tiled: Optional[torch.Tensor] =
     return linear(x, w, out_dtype, tiled=tiled, out=out)
 
 
-def linear_swiglu(x: torch.Tensor, w_gate_up: torch.Tensor, tiled: Optional[torch.Tensor] = None) -> torch.Tensor:
+def linear_swiglu(x: torch.Tensor, w_gate_up: torch.Tensor, tiled: Optional[torch.Tensor] = None, few_rows: int = 0) -> torch.Tensor:
     """silu(x . Wgate^T) * (x . Wup^T) with ``w_gate_up [2 I, K]`` = [Wgate | Wup] -> [M, I].  For few bfloat16 rows
-    (decode) one kernel does both products and the SwiGLU; otherwise it is linear() followed by swiglu()."""
+    (decode) one kernel does both products and the SwiGLU; otherwise it is linear() followed by swiglu().  ``few_rows``:
+    most rows that the tiled kernel takes here (0: SKINNY_MAX_ROWS)."""
     _dev(x, w_gate_up)
     _check(x.dim() == 2 and w_gate_up.dim() == 2 and x.shape[1] == w_gate_up.shape[1] and w_gate_up.shape[0] % 2 == 0,
            "linear_swiglu: x [M, K] and w [2 I, K] expected")
     M, K = x.shape
     I = w_gate_up.shape[0] // 2
-    if x.dtype == torch.bfloat16 and tiled is not None and 0 < M <= SKINNY_MAX_ROWS and I % 16 == 0:
+    if x.dtype == torch.bfloat16 and tiled is not None and 0 < M <= max(SKINNY_MAX_ROWS, few_rows) and I % 16 == 0 and x.is_contiguous():
         _check(tiled.shape == w_gate_up.shape, "linear_swiglu: the tiled copy does not fit")
         return decode_linear_swiglu(x, tiled)
     if x.dtype == torch.bfloat16 and w_gate_up.dtype == torch.bfloat16 and 0 < M <= SKINNY_MAX_ROWS and K % 8 == 0 \

@@ -240,6 +240,8 @@ class PagedAttention(Mixer):
         nq, nkv, d = self.num_heads, self.num_kv_heads, self.head_dim
         if isinstance(x, ops.ScaledInput):
             qkv = ops.decode_linear(x, self.w_qkv_tiled)
+        elif not self._plain_projections():
+            qkv = ops.linear_few(x, self.w_qkv, self.w_qkv_tiled)       # (no folded path here: the decode products up to 64 rows)
         else:
             qkv = ops.linear(x, self.w_qkv, tiled=self.w_qkv_tiled)
         meta = attention_meta(batch, cache.group, nq // nkv, self._big_rows(batch, cache.page_size))
@@ -274,6 +276,8 @@ class PagedAttention(Mixer):
                                    for_product=for_product)
 
     def forward(self, x, batch, cache, store=True):
+        if not self._plain_projections():
+            return ops.linear_few(self._attend(x, batch, cache, store), self.w_o, self.w_o_tiled)
         return ops.linear(self._attend(x, batch, cache, store), self.w_o, tiled=self.w_o_tiled)
 
     def forward_into(self, x, batch, cache, store, resid, next_norm):

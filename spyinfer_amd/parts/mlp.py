@@ -53,7 +53,8 @@ class GatedMLP(FeedForward):
     def forward(self, x, batch):
         if isinstance(x, ops.ScaledInput):
             return ops.linear(ops.decode_linear_swiglu(x, self.w_gate_up_tiled), self.w_down, tiled=self.w_down_tiled)
-        return ops.linear(ops.linear_swiglu(x, self.w_gate_up, self.w_gate_up_tiled), self.w_down, tiled=self.w_down_tiled)
+        return ops.linear_few(ops.linear_swiglu(x, self.w_gate_up, self.w_gate_up_tiled, few_rows=ops.DECODE_ROWS_PLAIN), self.w_down,
+                              self.w_down_tiled)
 
     def forward_into(self, x, batch, resid, next_norm):
         weight, eps = next_norm.foldable(batch.act_dtype)

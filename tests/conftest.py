@@ -32,7 +32,7 @@ def emu_ops(monkeypatch):
     monkeypatch.setattr(ops, "linear", linear)
     monkeypatch.setattr(ops, "linear_few", lambda x, w, tiled=None, out_dtype=None, out=None: linear(x, w, out_dtype, out=out))
     monkeypatch.setattr(ops, "linear_xielu", lambda x, w, pq, tiled=None: emu.xielu(emu.linear(x, w), pq))
-    monkeypatch.setattr(ops, "linear_swiglu", lambda x, w, tiled=None: emu.swiglu(emu.linear(x, w)))
+    monkeypatch.setattr(ops, "linear_swiglu", lambda x, w, tiled=None, few_rows=0: emu.swiglu(emu.linear(x, w)))
     monkeypatch.setattr(ops, "paged_attention", lambda q, k_cache, v_cache, page_size, meta, n_q, n_kv, d, scale, window, raw=None,
                         for_product=False: emu.paged_attention(q, k_cache, v_cache, page_size, meta, n_q, n_kv, d, scale, window))
     monkeypatch.setattr(ops, "latent_attention", lambda qa, cache, page_size, meta, sink, R, scale, window, out_dtype, tiles=None,

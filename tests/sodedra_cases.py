@@ -59,7 +59,7 @@ SOD_A = dict(architecture="Sodedra", vocab=97, width=48, norm=dict(eps=3e-6), em
 SOD_B = dict(architecture="Sodedra", vocab=61, width=32, norm=dict(eps=2e-5), embedding=dict(scale=1.0),
              layers=[_layer("channel_delta", _delta(1, 1, 8, 8, 1, 4, 4), _dense(32)),
                      _layer("attention", _attention(1, 1, 8, 8, 1.0, window=1, dims=8), _moe(32, 4, 1, 1, 1, 1.0)),
-                     _layer("mlstm", _mlstm(1, 8, 8, 15.0)),
+                     _layer("mlstm", _mlstm(1, 8, 8, 14.0)),
                      _layer("attention", _attention(4, 4, 8, 8, 0.5, window=2, dims=2, scaling=dict(factor=2.0, low=1.0, high=1.0, original=8)), _dense(32)),
                      _layer("channel_delta", _delta(2, 1, 8, 8, 2, 1, 1), _moe(8, 4, 4, 2, 2, 2.0))])
 
@@ -80,7 +80,7 @@ SOD_FAR = dict(architecture="Sodedra", vocab=83, width=40, norm=dict(eps=1e-6), 
 SOD_LONG = dict(architecture="Sodedra", vocab=211, width=64, norm=dict(eps=1e-6), embedding=dict(scale=0.9),
                 layers=[_layer("attention", _attention(4, 2, 16, 16, 0.3, window=333, base=50000.0, dims=12,
                                                        scaling=dict(factor=6.0, low=1.0, high=5.0, original=512)), _dense(96)),
-                        _layer("mlstm", _mlstm(2, 16, 24, 15.0), _moe(32, 6, 2, 3, 2, 1.2)),
+                        _layer("mlstm", _mlstm(2, 16, 24, 13.0), _moe(32, 6, 2, 3, 2, 1.2)),
                         _layer("channel_delta", _delta(2, 1, 16, 24, 4, 8, 8)),
                         _layer("attention", _attention(2, 2, 8, 24, 0.4, window=150, base=50000.0, dims=8), _dense(64))])
 

@@ -89,7 +89,7 @@ def test_norm_with_two_addends_and_scaled_embedding(dtype, T, H):
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
-@pytest.mark.parametrize("H,d,dv", [(3, 5, 7), (2, 48, 64), (2, 128, 96), (1, 200, 300), (2, 64, 600)])
+@pytest.mark.parametrize("H,d,dv", [(3, 5, 7), (2, 40, 72), (2, 128, 96), (1, 200, 300), (2, 64, 600)])
 def test_mlstm_carries_its_state_between_steps(dtype, H, d, dv):
     from spyinfer_amd.kernels import ops
     dev = require_gpu()
@@ -122,7 +122,7 @@ def test_mlstm_carries_its_state_between_steps(dtype, H, d, dv):
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
-@pytest.mark.parametrize("H,G,d,dv,taps", [(4, 2, 6, 5, 3), (2, 2, 64, 32, 4), (3, 1, 128, 128, 2), (1, 1, 40, 200, 1), (2, 1, 16, 8, 8)])
+@pytest.mark.parametrize("H,G,d,dv,taps", [(4, 2, 6, 5, 3), (2, 2, 56, 24, 4), (3, 1, 128, 128, 2), (1, 1, 40, 200, 1), (2, 1, 16, 8, 8)])
 def test_delta_rule_and_convolution_carry_their_state_between_steps(dtype, H, G, d, dv, taps):
     from spyinfer_amd.kernels import ops
     dev = require_gpu()
@@ -163,7 +163,7 @@ def test_delta_rule_and_convolution_carry_their_state_between_steps(dtype, H, G,
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
-@pytest.mark.parametrize("dims,scaling", [(8, None), (6, dict(factor=8.0, low=1.0, high=4.0, original=64)), (0, None), (24, dict(factor=4.0, low=1.0, high=4.0, original=1024))])
+@pytest.mark.parametrize("dims,scaling", [(8, None), (6, dict(factor=8.0, low=1.0, high=4.0, original=64)), (0, None), (20, dict(factor=5.0, low=1.0, high=3.0, original=2048))])
 def test_biases_rotation_and_store(dtype, dims, scaling):
     from spyinfer_amd.kernels import ops
     from spyinfer_amd.parts.rotary import RotaryEmbedding
@@ -199,7 +199,7 @@ def test_biases_rotation_and_store(dtype, dims, scaling):
     close(ops.sigmoid_gate(y.to(dev), wide.to(dev)[:, 9:33]), y.double() * torch.sigmoid(wide.double()[:, 9:33]), DT[dtype], what="gate")
 
 
-@pytest.mark.parametrize("E,top,groups,keep", [(12, 4, 4, 3), (8, 3, 4, 2), (4, 1, 1, 1), (64, 8, 8, 4), (6, 6, 3, 3), (130, 5, 10, 2)])
+@pytest.mark.parametrize("E,top,groups,keep", [(12, 3, 3, 2), (8, 3, 4, 2), (4, 1, 1, 1), (64, 8, 8, 4), (6, 6, 3, 3), (130, 5, 10, 2)])
 def test_router_chooses_among_the_best_groups(E, top, groups, keep):
     from spyinfer_amd.kernels import ops
     dev = require_gpu()
