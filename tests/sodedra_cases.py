@@ -84,6 +84,11 @@ SOD_LONG = dict(architecture="Sodedra", vocab=211, width=64, norm=dict(eps=1e-6)
                         _layer("channel_delta", _delta(2, 1, 16, 24, 4, 8, 8)),
                         _layer("attention", _attention(2, 2, 8, 24, 0.4, window=150, base=50000.0, dims=8), _dense(64))])
 
+#: no attention layer at all: no page group, only state slots
+SOD_REC = dict(architecture="Sodedra", vocab=53, width=24, norm=dict(eps=1e-5), embedding=dict(scale=1.2),
+               layers=[_layer("mlstm", _mlstm(2, 4, 6, 9.0), _dense(32)),
+                       _layer("channel_delta", _delta(2, 1, 4, 6, 3, 3, 3), _moe(8, 4, 2, 2, 1, 1.1))])
+
 INIT = dict(matrix_std=0.12, norm_std=0.2, bias_std=0.3)
 
 

@@ -264,6 +264,18 @@ def test_schedules_equal_the_plain_implementation(folders, name, mode, dtype, tm
     compare(rc.collect(str(tmp_path), steps, sc.vocab_of(folder)), sc.plain_logits(folder, requests), dtype, "%s/%s/%s" % (name, mode, dtype))
 
 
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_recurrences_alone_run_without_any_page_group(dtype, tmp_path):
+    require_gpu()
+    folder = sc.write_model(str(tmp_path / "m"), sc.SOD_REC, 1, None)
+    requests = rc.random_requests(53, [21, 1, 2, 33, 9], 5)
+    ref = sc.plain_logits(folder, requests)
+    for name, steps in (("whole", rc.whole(requests)), ("portions", rc.portions(requests)), ("mixed", rc.mixed(requests))):
+        out = str(tmp_path / name)
+        rc.run_replay_inprocess(folder, dtype, out, steps, rc.max_live_tokens(steps), ["--poison-cache"])
+        compare(rc.collect(out, steps, 53), ref, dtype, "recurrences alone/%s/%s" % (name, dtype))
+
+
 @pytest.mark.parametrize("mode", ["whole", "bulk_tail", "portions"])
 def test_far_keys_among_hundreds(folders, mode, tmp_path):
     """One attention layer without a window and with sharp scores: the keys that decide a row's result lie anywhere in

@@ -88,6 +88,16 @@ def test_schedules_equal_the_plain_implementation(folders, name, mode, tmp_path,
     rc.compare(rc.collect(str(tmp_path), steps, sc.vocab_of(folder)), sc.plain_logits(folder, requests), what="%s/%s" % (name, mode), **TOL)
 
 
+def test_recurrences_alone_run_without_any_page_group(tmp_path, emu_ops):
+    folder = sc.write_model(str(tmp_path / "m"), sc.SOD_REC, 1, None, torch.float32)
+    requests = rc.random_requests(53, [21, 1, 2, 33, 9], 5)
+    ref = sc.plain_logits(folder, requests)
+    for name, steps in (("whole", rc.whole(requests)), ("portions", rc.portions(requests)), ("mixed", rc.mixed(requests))):
+        out = str(tmp_path / name)
+        rc.run_replay_inprocess(folder, "float32", out, steps, rc.max_live_tokens(steps), CPU)
+        rc.compare(rc.collect(out, steps, 53), ref, what=name, **TOL)
+
+
 def test_pages_of_passed_windows_and_slots_go_back_and_are_used_again(folders, emu_ops):
     from spyinfer_amd.engine.batch import StepEntry
     from spyinfer_amd.engine.runner import ModelRunner, load_model
