@@ -21,8 +21,7 @@ __device__ __forceinline__ float mm_logsigmoid(float x) { return fminf(x, 0.f) -
 #define MM_COLS 16           // value channels of a wave: four lanes a column
 
 // Between a wave's LDS writes and its own LDS reads: a block here is ONE wave, whose LDS operations run in program order,
-// so no barrier is needed, and none is wanted: a barrier would also wait for the global loads that are in flight for
-// the tokens ahead.  What is needed is that the compiler keeps the order.
+// so no barrier is needed.  What is needed is that the compiler keeps the order.
 __device__ __forceinline__ void mm_wave_order() {
     __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
     __builtin_amdgcn_wave_barrier();
