@@ -334,7 +334,8 @@ class SodedraConfig(ModelConfig):
             mix = {k: _need(m, k, int, at) for k in ("heads", "dim", "vdim")}
             mix["gate_cap"] = float(_need(m, "gate_cap", (int, float), at))
         elif kind == "attention":
-            mix = {k: _need(m, k, int, at) for k in ("heads", "kv_heads", "dim", "vdim")}
+            mix = {k: _need(m, k, int, at) for k in ("heads", "dim", "vdim")}
+            mix["kv_heads"] = _need(m, "kv_heads", int, at) if m.get("kv_heads") is not None else mix["heads"]
             mix["scale"] = float(_need(m, "scale", (int, float), at))
             mix["window"] = _need(m, "mask.size", int, at) if m.get("mask") else None
             rot = m.get("rot")
@@ -346,7 +347,8 @@ class SodedraConfig(ModelConfig):
                 if sc:
                     mix["rot"]["scaling"] = {k: float(_need(sc, k, (int, float), at + ".rot.scaling")) for k in ("factor", "low", "high", "original")}
         else:
-            mix = {k: _need(m, k, int, at) for k in ("heads", "kv_heads", "dim", "vdim", "conv")}
+            mix = {k: _need(m, k, int, at) for k in ("heads", "dim", "vdim", "conv")}
+            mix["kv_heads"] = _need(m, "kv_heads", int, at) if m.get("kv_heads") is not None else mix["heads"]
             # inner sizes of the low-rank projections: no key of the design; the stored tensors decide unless these are given
             for k in ("decay_rank", "gate_rank"):
                 mix[k] = _need(m, k, int, at) if m.get(k) is not None else None
