@@ -72,14 +72,25 @@ __global__ void mlstm_gates_kernel(float* __restrict__ gates, const TW* __restri
 // S (row dd, column j at dd dv + j), then for every slice of 16 columns its own copy of n and m (the slices' waves do
 // not wait for each other, so none may read what another has already moved on).
 #define MM_AHEAD 4          // tokens whose operands are in flight ahead of the one being worked on
-template <typename TA, typename TW, int DR>
+// MODE 0: block x is an entry, walked whole from the request's state, which is left at the end.
+// Entries of many tokens are cut into pieces (block x is a piece then): with the running maximum known for every token
+// (mlstm_scalars_kernel: a, b and exp(-m) per token in `gates` [T, 3 H]) the state is linear in itself with scalar
+// coefficients, S_end = A S_start + B with A the product of the piece's a.  MODE 1 walks a piece from zero and leaves
+// (B, A) in the piece's record of `work` (laid out as a request's state, A where m lies); MODE 2 folds the records of
+// the entry's pieces before its own into the request's state, walks its piece from there and writes the read-outs;
+// mlstm_keep_kernel folds all of an entry's records into the state afterwards.
+template <typename TA, typename TW, int DR, int MODE>
 __global__ __launch_bounds__(MM_SLICE) void mlstm_kernel(
     float* __restrict__ o_out, float* __restrict__ state, const TA* __restrict__ x, long long xs, int q_off, int k_off, int v_off,
     const float* __restrict__ gates, const int* __restrict__ cu_q,
-    const int* __restrict__ slot_ids, int num_slots, int H, int d, int dv, int NS) {
+    const int* __restrict__ slot_ids, int num_slots, int H, int d, int dv, int NS,
+    float* __restrict__ work, const int* __restrict__ piece_entry, const int* __restrict__ piece_t0, const int* __restrict__ piece_t1,
+    const int* __restrict__ piece_first) {
     constexpr int R = (DR + MM_SLICE - 1) / MM_SLICE, LD = R * MM_SLICE, DQ = DR / 4;
+    constexpr int GS = MODE == 0 ? 2 : 3;             // scalars a token and head in `gates`
     __shared__ __align__(16) float ks[LD], qs[LD];
-    const int s = blockIdx.x, h = blockIdx.y, c = blockIdx.z, lane = threadIdx.x;
+    const int h = blockIdx.y, c = blockIdx.z, lane = threadIdx.x;
+    const int s = MODE == 0 ? (int)blockIdx.x : piece_entry[blockIdx.x];
     const int part = lane & 3, j = c * MM_COLS + (lane >> 2);
     const int row0 = part * DQ;                       // this lane's rows of S: row0 .. row0 + DQ - 1
     const int slot = slot_ids[s];
@@ -93,18 +104,41 @@ __global__ __launch_bounds__(MM_SLICE) void mlstm_kernel(
     float S[DQ], n[DQ];
 #pragma unroll
     for (int i = 0; i < DQ; ++i) {
-        S[i] = (col && row0 + i < d) ? st[(size_t)(row0 + i) * dv + j] : 0.f;
-        n[i] = row0 + i < d ? nm[row0 + i] : 0.f;
+        S[i] = (MODE != 1 && col && row0 + i < d) ? st[(size_t)(row0 + i) * dv + j] : 0.f;
+        n[i] = (MODE != 1 && row0 + i < d) ? nm[row0 + i] : 0.f;
+    }
+    if (MODE == 2) {
+        const int jc = min(j, dv - 1);
+        for (int q = piece_first[blockIdx.x]; q < (int)blockIdx.x; ++q) {
+            const float* ws = work + ((size_t)q * H + h) * head_state;
+            const float* wn = ws + (size_t)d * dv + (size_t)c * (d + 1);
+            const float A = wn[d];
+            // (loads without conditions, from clamped places, so that they all go out together; rows and columns that do
+            // not exist keep their zeros)
+            float ws_[DQ], wn_[DQ];
+#pragma unroll
+            for (int i = 0; i < DQ; ++i) {
+                ws_[i] = ws[(size_t)min(row0 + i, d - 1) * dv + jc];
+                wn_[i] = wn[min(row0 + i, d - 1)];
+            }
+#pragma unroll
+            for (int i = 0; i < DQ; ++i) {
+                const bool rok = row0 + i < d;
+                S[i] = (col && rok) ? fmaf(A, S[i], ws_[i]) : S[i];
+                n[i] = rok ? fmaf(A, n[i], wn_[i]) : n[i];
+            }
+        }
     }
 #pragma unroll
     for (int i = 0; i < R; ++i) {
         ks[lane + MM_SLICE * i] = 0.f;
         qs[lane + MM_SLICE * i] = 0.f;
     }
-    float m = nm[d];
+    float m = MODE == 0 ? nm[d] : 0.f;
+    float Aprod = 1.f;
     const float qscale = 1.0f / sqrtf((float)d);
-    const int t0 = cu_q[s], t1 = cu_q[s + 1];
-    float kr[MM_AHEAD][R], qr[MM_AHEAD][R], vr[MM_AHEAD], gir[MM_AHEAD], gfr[MM_AHEAD];
+    const int t0 = MODE == 0 ? cu_q[s] : piece_t0[blockIdx.x], t1 = MODE == 0 ? cu_q[s + 1] : piece_t1[blockIdx.x];
+    float kr[MM_AHEAD][R], qr[MM_AHEAD][R], vr[MM_AHEAD], gir[MM_AHEAD], gfr[MM_AHEAD], ger[MM_AHEAD];
 #define MLSTM_LOAD(U, TT)                                                                        \
     if ((TT) < t1) {                                                                             \
         const TA* xr_ = x + (size_t)(TT) * xs;                                                   \
@@ -114,8 +148,9 @@ __global__ __launch_bounds__(MM_SLICE) void mlstm_kernel(
             qr[U][i] = idx < d ? to_f32<TA>(xr_[q_off + (size_t)h * d + idx]) * qscale : 0.f;    \
         }                                                                                        \
         vr[U] = col ? to_f32<TA>(xr_[v_off + (size_t)h * dv + j]) : 0.f;                         \
-        gir[U] = gates[(size_t)(TT) * 2 * H + h];                                                \
-        gfr[U] = gates[(size_t)(TT) * 2 * H + H + h];                                            \
+        gir[U] = gates[(size_t)(TT) * GS * H + h];                                               \
+        gfr[U] = gates[(size_t)(TT) * GS * H + H + h];                                           \
+        ger[U] = MODE == 0 ? 0.f : gates[(size_t)(TT) * GS * H + 2 * H + h];                     \
     }
 #pragma unroll
     for (int u = 0; u < MM_AHEAD; ++u) MLSTM_LOAD(u, t0 + u)
@@ -129,10 +164,20 @@ __global__ __launch_bounds__(MM_SLICE) void mlstm_kernel(
                     const int idx = lane + MM_SLICE * i;
                     if (idx < d) { ks[idx] = kr[u][i]; qs[idx] = qr[u][i]; }
                 }
-                const float ig = gir[u], fg = gfr[u];
-                const float m_new = fmaxf(fg + m, ig);
-                const float a = expf(fg + m - m_new), b = expf(ig - m_new);
-                m = m_new;
+                float a, b, em;
+                if (MODE == 0) {
+                    const float ig = gir[u], fg = gfr[u];
+                    const float m_new = fmaxf(fg + m, ig);
+                    a = expf(fg + m - m_new);
+                    b = expf(ig - m_new);
+                    m = m_new;
+                    em = expf(-m);
+                } else {
+                    a = gir[u];
+                    b = gfr[u];
+                    em = ger[u];
+                    Aprod *= a;
+                }
                 mm_wave_order();
                 float acc = 0.f, acc2 = 0.f, nq = 0.f, nq2 = 0.f;
                 const float bv = b * vr[u];
@@ -150,20 +195,125 @@ __global__ __launch_bounds__(MM_SLICE) void mlstm_kernel(
                 }
                 acc = quad_sum(acc + acc2);
                 nq = quad_sum(nq + nq2);
-                const float den = fmaxf(fabsf(nq), expf(-m)) + 1e-6f;
-                if (col && part == 0) o_out[((size_t)t * H + h) * dv + j] = acc / den;
+                const float den = fmaxf(fabsf(nq), em) + 1e-6f;
+                if (MODE != 1 && col && part == 0) o_out[((size_t)t * H + h) * dv + j] = acc / den;
                 mm_wave_order();
                 MLSTM_LOAD(u, t + MM_AHEAD)
             }
         }
     }
 #undef MLSTM_LOAD
+    if (MODE == 2) return;
+    if (MODE == 1) {
+        st = work + ((size_t)blockIdx.x * H + h) * head_state;
+        nm = st + (size_t)d * dv + (size_t)c * (d + 1);
+        m = Aprod;
+    }
 #pragma unroll
     for (int i = 0; i < DQ; ++i) {
         if (col && row0 + i < d) st[(size_t)(row0 + i) * dv + j] = S[i];
         if (lane < 4 && row0 + i < d) nm[row0 + i] = n[i];
     }
     if (lane == 0) nm[d] = m;
+}
+
+// One thread per (entry, head): the running maximum over the entry's tokens, from the request's state, before and after
+// every token in abe [T, 3 H]; the last maximum goes to mfin [S, H].
+__global__ void mlstm_scalars_kernel(float* __restrict__ abe, float* __restrict__ mfin, const float* __restrict__ lg,
+                                     const float* __restrict__ state, const int* __restrict__ cu_q, const int* __restrict__ slot_ids,
+                                     int num_slots, int S, int H, int d, int dv, int NS) {
+    const int i = blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= S * H) return;
+    const int s = i / H, h = i - s * H;
+    const int slot = slot_ids[s];
+    if (slot < 0 || slot >= num_slots) return;
+    const size_t head_state = (size_t)d * dv + (size_t)NS * (d + 1);
+    float m = state[((size_t)slot * H + h) * head_state + (size_t)d * dv + d];
+    const int t1 = cu_q[s + 1];
+    // (the gates of 16 tokens are asked for together: the loads do not depend on the maximum, only the arithmetic does)
+    for (int tb = cu_q[s]; tb < t1; tb += 16) {
+        float ig[16], fg[16];
+#pragma unroll
+        for (int u = 0; u < 16; ++u) {
+            const int t = tb + u < t1 ? tb + u : t1 - 1;
+            ig[u] = lg[(size_t)t * 2 * H + h];
+            fg[u] = lg[(size_t)t * 2 * H + H + h];
+        }
+#pragma unroll
+        for (int u = 0; u < 16; ++u) {
+            const int t = tb + u;
+            if (t < t1) {
+                const float m_new = fmaxf(fg[u] + m, ig[u]);
+                abe[(size_t)t * 3 * H + h] = m;                      // (the exponentials follow for all tokens at once)
+                abe[(size_t)t * 3 * H + H + h] = m_new;
+                m = m_new;
+            }
+        }
+    }
+    mfin[i] = m;
+}
+
+// abe [T, 3 H] holds the maximum before and after every token (mlstm_scalars_kernel); with the log gates lg [T, 2 H] it
+// becomes a = exp(f + m' - m), b = exp(i - m) and exp(-m).
+__global__ void mlstm_abe_kernel(float* __restrict__ abe, const float* __restrict__ lg, int T, int H) {
+    const size_t total = (size_t)T * H;
+    for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < total; i += (size_t)gridDim.x * blockDim.x) {
+        const size_t t = i / H, h = i - t * H;
+        const float mp = abe[t * 3 * H + h], mn = abe[t * 3 * H + H + h];
+        const float ig = lg[t * 2 * H + h], fg = lg[t * 2 * H + H + h];
+        abe[t * 3 * H + h] = expf(fg + mp - mn);
+        abe[t * 3 * H + H + h] = expf(ig - mn);
+        abe[t * 3 * H + 2 * H + h] = expf(-mn);
+    }
+}
+
+// Block x is a piece; the last piece of an entry folds all of the entry's records into the request's state.
+template <int DR>
+__global__ __launch_bounds__(MM_SLICE) void mlstm_keep_kernel(float* __restrict__ state, const float* __restrict__ work,
+                                                              const float* __restrict__ mfin, const int* __restrict__ piece_entry,
+                                                              const int* __restrict__ piece_first, int n_pieces,
+                                                              const int* __restrict__ slot_ids, int num_slots, int H, int d, int dv, int NS) {
+    constexpr int DQ = DR / 4;
+    const int k = blockIdx.x, h = blockIdx.y, c = blockIdx.z, lane = threadIdx.x;
+    if (!(k + 1 == n_pieces || piece_first[k + 1] == k + 1)) return;
+    const int s = piece_entry[k];
+    const int slot = slot_ids[s];
+    if (slot < 0 || slot >= num_slots) return;
+    const int part = lane & 3, j = c * MM_COLS + (lane >> 2), row0 = part * DQ;
+    const bool col = j < dv;
+    const size_t head_state = (size_t)d * dv + (size_t)NS * (d + 1);
+    float* st = state + ((size_t)slot * H + h) * head_state;
+    float* nm = st + (size_t)d * dv + (size_t)c * (d + 1);
+    float S[DQ], n[DQ];
+#pragma unroll
+    for (int i = 0; i < DQ; ++i) {
+        S[i] = (col && row0 + i < d) ? st[(size_t)(row0 + i) * dv + j] : 0.f;
+        n[i] = row0 + i < d ? nm[row0 + i] : 0.f;
+    }
+    const int jc = min(j, dv - 1);
+    for (int q = piece_first[k]; q <= k; ++q) {
+        const float* ws = work + ((size_t)q * H + h) * head_state;
+        const float* wn = ws + (size_t)d * dv + (size_t)c * (d + 1);
+        const float A = wn[d];
+        float ws_[DQ], wn_[DQ];
+#pragma unroll
+        for (int i = 0; i < DQ; ++i) {
+            ws_[i] = ws[(size_t)min(row0 + i, d - 1) * dv + jc];
+            wn_[i] = wn[min(row0 + i, d - 1)];
+        }
+#pragma unroll
+        for (int i = 0; i < DQ; ++i) {
+            const bool rok = row0 + i < d;
+            S[i] = (col && rok) ? fmaf(A, S[i], ws_[i]) : S[i];
+            n[i] = rok ? fmaf(A, n[i], wn_[i]) : n[i];
+        }
+    }
+#pragma unroll
+    for (int i = 0; i < DQ; ++i) {
+        if (col && row0 + i < d) st[(size_t)(row0 + i) * dv + j] = S[i];
+        if (lane < 4 && row0 + i < d) nm[row0 + i] = n[i];
+    }
+    if (lane == 0) nm[d] = mfin[(size_t)s * H + h];
 }
 
 #define MM_LAUNCH(KERNEL, ...)                                                              \
@@ -174,9 +324,20 @@ __global__ __launch_bounds__(MM_SLICE) void mlstm_kernel(
         else KERNEL<TA, TW, 256><<<grid, MM_SLICE, 0, st>>>(__VA_ARGS__);                   \
     } while (0)
 
+#define MM_LAUNCH_MODE(KERNEL, MODE, ...)                                                          \
+    do {                                                                                           \
+        if (d <= 32) KERNEL<TA, TW, 32, MODE><<<grid, MM_SLICE, 0, st>>>(__VA_ARGS__);             \
+        else if (d <= 64) KERNEL<TA, TW, 64, MODE><<<grid, MM_SLICE, 0, st>>>(__VA_ARGS__);        \
+        else if (d <= 128) KERNEL<TA, TW, 128, MODE><<<grid, MM_SLICE, 0, st>>>(__VA_ARGS__);      \
+        else KERNEL<TA, TW, 256, MODE><<<grid, MM_SLICE, 0, st>>>(__VA_ARGS__);                    \
+    } while (0)
+
+// pieces: int32 [4][n_pieces] (entry, first row, end row, index of the entry's first piece), used when `multi` says that an
+// entry has several; then work [n_pieces][state of a request], abe [T][3 H] and mfin [S][H] are scratch.
 extern "C" int spy_mlstm(void* out, float* o_tmp, float* state, const void* x, long long xs, int dtype, int q_off, int k_off, int v_off,
                          int g_off, float* gates, const void* bi, const void* bf, int w_dtype, float cap, const void* norm_w,
-                         float eps, const int* cu_q, const int* slot_ids, int num_slots, int S, int T, int H, int d, int dv, hipStream_t st) {
+                         float eps, const int* cu_q, const int* slot_ids, int num_slots, int S, int T, int H, int d, int dv,
+                         const int* pieces, int n_pieces, int multi, float* work, float* abe, float* mfin, hipStream_t st) {
     SPY_REQUIRE(S > 0 && T > 0 && H > 0 && d > 0 && dv > 0 && num_slots > 0 && o_tmp, "spy_mlstm: empty operand");
     SPY_REQUIRE(d <= 256 && dv <= 1024 && H <= 65535, "spy_mlstm: heads of %d x %d (key size up to 256, value size up to 1024)", d, dv);
     SPY_REQUIRE(cap > 0.f, "spy_mlstm: the gates' cap must be positive");
@@ -188,9 +349,37 @@ extern "C" int spy_mlstm(void* out, float* o_tmp, float* state, const void* x, l
         SPY_DISPATCH(w_dtype, TW, (mlstm_gates_kernel<TW><<<blocks, 256, 0, st>>>(gates, (const TW*)bi, (const TW*)bf, cap, T, H)));
         SPY_CHECK_LAUNCH("spy_mlstm (gates)");
     }
-    SPY_DISPATCH(dtype, TA, SPY_DISPATCH(w_dtype, TW, MM_LAUNCH(mlstm_kernel, o_tmp, state, (const TA*)x, xs, q_off, k_off, v_off, gates,
-        cu_q, slot_ids, num_slots, H, d, dv, NS)));
-    SPY_CHECK_LAUNCH("spy_mlstm");
+    if (!multi) {
+        SPY_DISPATCH(dtype, TA, SPY_DISPATCH(w_dtype, TW, MM_LAUNCH_MODE(mlstm_kernel, 0, o_tmp, state, (const TA*)x, xs, q_off, k_off, v_off,
+            gates, cu_q, slot_ids, num_slots, H, d, dv, NS, nullptr, nullptr, nullptr, nullptr, nullptr)));
+        SPY_CHECK_LAUNCH("spy_mlstm");
+    } else {
+        SPY_REQUIRE(pieces && n_pieces > 0 && work && abe && mfin, "spy_mlstm: entries in several pieces need their scratch memory");
+        const int* pe = pieces;
+        const int* p0 = pieces + n_pieces;
+        const int* p1 = pieces + 2 * (size_t)n_pieces;
+        const int* pf = pieces + 3 * (size_t)n_pieces;
+        mlstm_scalars_kernel<<<(S * H + 63) / 64, 64, 0, st>>>(abe, mfin, gates, state, cu_q, slot_ids, num_slots, S, H, d, dv, NS);
+        SPY_CHECK_LAUNCH("spy_mlstm (running maximum)");
+        {
+            const size_t total = (size_t)T * H;
+            const unsigned blocks = (unsigned)((total + 255) / 256 > 4096 ? 4096 : (total + 255) / 256);
+            mlstm_abe_kernel<<<blocks, 256, 0, st>>>(abe, gates, T, H);
+            SPY_CHECK_LAUNCH("spy_mlstm (decays)");
+        }
+        const dim3 grid(n_pieces, H, NS);
+        SPY_DISPATCH(dtype, TA, SPY_DISPATCH(w_dtype, TW, MM_LAUNCH_MODE(mlstm_kernel, 1, o_tmp, state, (const TA*)x, xs, q_off, k_off, v_off,
+            abe, cu_q, slot_ids, num_slots, H, d, dv, NS, work, pe, p0, p1, pf)));
+        SPY_CHECK_LAUNCH("spy_mlstm (pieces)");
+        SPY_DISPATCH(dtype, TA, SPY_DISPATCH(w_dtype, TW, MM_LAUNCH_MODE(mlstm_kernel, 2, o_tmp, state, (const TA*)x, xs, q_off, k_off, v_off,
+            abe, cu_q, slot_ids, num_slots, H, d, dv, NS, work, pe, p0, p1, pf)));
+        SPY_CHECK_LAUNCH("spy_mlstm (walk)");
+        if (d <= 32) mlstm_keep_kernel<32><<<grid, MM_SLICE, 0, st>>>(state, work, mfin, pe, pf, n_pieces, slot_ids, num_slots, H, d, dv, NS);
+        else if (d <= 64) mlstm_keep_kernel<64><<<grid, MM_SLICE, 0, st>>>(state, work, mfin, pe, pf, n_pieces, slot_ids, num_slots, H, d, dv, NS);
+        else if (d <= 128) mlstm_keep_kernel<128><<<grid, MM_SLICE, 0, st>>>(state, work, mfin, pe, pf, n_pieces, slot_ids, num_slots, H, d, dv, NS);
+        else mlstm_keep_kernel<256><<<grid, MM_SLICE, 0, st>>>(state, work, mfin, pe, pf, n_pieces, slot_ids, num_slots, H, d, dv, NS);
+        SPY_CHECK_LAUNCH("spy_mlstm (state)");
+    }
     const dim3 ngrid(T, H);
     const int nthreads = dv >= 256 ? 256 : 64;
     SPY_DISPATCH(dtype, TA, SPY_DISPATCH(w_dtype, TW, (head_norm_gate_kernel<TA, TW><<<ngrid, nthreads, 0, st>>>(

@@ -1210,13 +1210,15 @@ def _entries(cu_q: torch.Tensor, slot_ids: torch.Tensor, what: str) -> int:
 
 def mlstm(x: torch.Tensor, q_off: int, k_off: int, v_off: int, g_off: int, gates: torch.Tensor, bi: torch.Tensor, bf: torch.Tensor,
           cap: float, norm_w: torch.Tensor, eps: float, state: torch.Tensor, cu_q: torch.Tensor, slot_ids: torch.Tensor, H: int, d: int,
-          dv: int) -> torch.Tensor:
+          dv: int, pieces=None) -> torch.Tensor:
     """The mLSTM recurrence over the step's tokens.  ``x``: rows of the fused projection with q (H heads of d) at column
     ``q_off``, k at ``k_off``, v (H heads of dv) at ``v_off`` and the output gate's rows at ``g_off``; ``gates [T, 2 H]``
     float32: the raw products of the input and forget gates, overwritten with the log gates (their biases ``bi``, ``bf [H]``; both capped by
     cap tanh(. / cap)); ``state [slots, mlstm_state_size(H, d, dv)]`` float32 holds S, n and the running maximum of every
-    head, read at an entry's start and left at its end.  Returns [T, H dv]: each head's read-out over its root mean square, times
-    ``norm_w``, times sigmoid(gate)."""
+    head, read at an entry's start and left at its end.  ``pieces`` = (int32 [4 n]: entry, first row, end row and the
+    entry's first piece for every piece of tokens; n; whether an entry has several): entries in several pieces are walked
+    by several waves, whose effects on the state are composed.  Returns [T, H dv]: each head's read-out over its root
+    mean square, times ``norm_w``, times sigmoid(gate)."""
     xs = _row_view(x, "mlstm")
     T = x.shape[0]
     _dev(gates, bi, bf, norm_w, state, cu_q, slot_ids)
@@ -1233,10 +1235,19 @@ def mlstm(x: torch.Tensor, q_off: int, k_off: int, v_off: int, g_off: int, gates
     out = torch.empty((T, H * dv), dtype=x.dtype, device=x.device)
     if T:
         tmp = torch.empty((T, H * dv), dtype=torch.float32, device=x.device)        # the read-outs before the heads' norm
+        parr, n_pieces, multi, work, abe, mfin = None, 0, False, None, None, None
+        if pieces is not None and pieces[2]:
+            parr, n_pieces, multi = pieces
+            _dev(parr)
+            _check(parr.dtype == torch.int32 and parr.shape == (4 * n_pieces,) and n_pieces > 0, "mlstm: pieces must be int32 [4 n]")
+            work = torch.empty((n_pieces, state.shape[1]), dtype=torch.float32, device=x.device)
+            abe = torch.empty((T, 3 * H), dtype=torch.float32, device=x.device)
+            mfin = torch.empty((S, H), dtype=torch.float32, device=x.device)
         hip().call("spy_mlstm", _ptr(out), _ptr(tmp), _ptr(state), ctypes.c_void_p(x.data_ptr()), ctypes.c_longlong(xs), _code(x, "x"), ctypes.c_int(q_off),
                    ctypes.c_int(k_off), ctypes.c_int(v_off), ctypes.c_int(g_off), _ptr(gates), _ptr(bi), _ptr(bf), _code(bi, "gate biases"),
                    ctypes.c_float(cap), _ptr(norm_w), ctypes.c_float(eps), _ptr(cu_q), _ptr(slot_ids), ctypes.c_int(state.shape[0]),
-                   ctypes.c_int(S), ctypes.c_int(T), ctypes.c_int(H), ctypes.c_int(d), ctypes.c_int(dv), _Hip.stream())
+                   ctypes.c_int(S), ctypes.c_int(T), ctypes.c_int(H), ctypes.c_int(d), ctypes.c_int(dv), _ptr(parr), ctypes.c_int(n_pieces),
+                   ctypes.c_int(1 if multi else 0), _ptr(work), _ptr(abe), _ptr(mfin), _Hip.stream())
     return out
 
 

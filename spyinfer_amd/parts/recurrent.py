@@ -31,10 +31,15 @@ from .base import Mixer
 SCAN_PIECE = 32
 
 
+def scan_pieces_name(piece: int = SCAN_PIECE) -> str:
+    return "scan_pieces" if piece == SCAN_PIECE else "scan_pieces_%d" % piece
+
+
 def plan_scan_pieces(batch, piece: int = SCAN_PIECE) -> None:
     """Adds the step's entries cut into pieces of at most ``piece`` tokens: int32 [4 n] = entry, first row, end row,
-    index of the entry's first piece.  Once per step."""
-    if "scan_pieces" in batch.shared:
+    index of the entry's first piece.  Once per step and piece size (``scan_pieces_name``)."""
+    name = scan_pieces_name(piece)
+    if name in batch.shared:
         return
     lens = batch.lens.astype(np.int64)
     cu = batch.host_array("cu_q").astype(np.int64)
@@ -46,8 +51,8 @@ def plan_scan_pieces(batch, piece: int = SCAN_PIECE) -> None:
     k = np.arange(n, dtype=np.int64) - first[:-1][entry]
     t0 = cu[:-1][entry] + k * piece
     t1 = np.minimum(t0 + piece, cu[1:][entry])
-    batch.add_array("scan_pieces", np.concatenate([entry, t0, t1, first[:-1][entry]]).astype(np.int32))
-    batch.shared["scan_pieces"] = (n, bool((counts > 1).any()))
+    batch.add_array(name, np.concatenate([entry, t0, t1, first[:-1][entry]]).astype(np.int32))
+    batch.shared[name] = (n, bool((counts > 1).any()))
 
 
 class MinGRU(Mixer):
@@ -133,6 +138,16 @@ class MLSTM(Mixer):
     def cache_spec(self):
         return FixedState((ops.mlstm_state_size(self.heads, self.dim, self.vdim),), "float32")
 
+    #: tokens of an entry that one wave walks in a row; longer entries are cut (their pieces' effects on the state are
+    #: composed: with the running maximum known, the state is linear in itself)
+    PIECE = 64
+
+    def plan(self, batch) -> None:
+        plan_scan_pieces(batch, self.PIECE)
+
+    def plan_arrays(self, entries):
+        return {scan_pieces_name(self.PIECE): 4 * entries}
+
     def capturable(self, batch):
         return True
 
@@ -142,8 +157,10 @@ class MLSTM(Mixer):
         H, d, dv = self.heads, self.dim, self.vdim
         proj = ops.linear_few(x, self.w_in, self.w_in_tiled)
         gates = ops.linear(x, self.w_gates, torch.float32)
+        name = scan_pieces_name(self.PIECE)
+        n, multi = batch.shared[name]
         y = ops.mlstm(proj, 0, H * d, 2 * H * d, 2 * H * d + H * dv, gates, self.b_i, self.b_f, self.gate_cap, self.norm, self.norm_eps,
-                      cache.state, batch.array("cu_q"), batch.array("slot_ids"), H, d, dv)
+                      cache.state, batch.array("cu_q"), batch.array("slot_ids"), H, d, dv, pieces=(batch.array(name), n, multi))
         return ops.linear_few(y, self.w_o, self.w_o_tiled)
 
 

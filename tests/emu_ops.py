@@ -242,7 +242,7 @@ class EmuOps:
         return y
 
     # ---- matrix memories ----
-    def mlstm(self, x, q_off, k_off, v_off, g_off, gates, bi, bf, cap, norm_w, eps, state, cu_q, slot_ids, H, d, dv):
+    def mlstm(self, x, q_off, k_off, v_off, g_off, gates, bi, bf, cap, norm_w, eps, state, cu_q, slot_ids, H, d, dv, pieces=None):
         T = x.shape[0]
         f = x.float()
         out = torch.zeros((T, H, dv), dtype=torch.float32)

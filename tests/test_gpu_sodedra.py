@@ -88,13 +88,22 @@ def test_norm_with_two_addends_and_scaled_embedding(dtype, T, H):
     close(ops.embedding(i32(ids.tolist(), dev), table.to(dev), 0.37), table.double()[ids] * 0.37, torch.float32, what="scaled embedding")
 
 
+def scan_pieces(cu, piece):
+    """The pieces of a step's entries as the engine plans them: int32 [4 n] and whether an entry has several."""
+    rec = [(e, t, min(t + piece, cu[e + 1])) for e in range(len(cu) - 1) for t in range(cu[e], cu[e + 1], piece)]
+    first = [min(k for k, r in enumerate(rec) if r[0] == e) for e, _, _ in rec]
+    return [r[0] for r in rec] + [r[1] for r in rec] + [r[2] for r in rec] + first, len(rec), len(rec) > len(cu) - 1
+
+
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("lengths,cut,piece", [([37, 9, 1], [20, 1, 0], 0), ([150, 70, 1], [100, 64, 0], 64), ([37, 9, 2], [20, 1, 1], 4)])
 @pytest.mark.parametrize("H,d,dv", [(3, 5, 7), (2, 40, 72), (2, 128, 96), (1, 200, 300), (2, 64, 600)])
-def test_mlstm_carries_its_state_between_steps(dtype, H, d, dv):
+def test_mlstm_carries_its_state_between_steps(dtype, H, d, dv, lengths, cut, piece):
+    """``piece`` > 0: entries are cut into pieces of that many tokens, walked by different waves and composed."""
     from spyinfer_amd.kernels import ops
     dev = require_gpu()
     g = torch.Generator().manual_seed(3)
-    lengths, cut, cap, eps = [37, 9, 1], [20, 1, 0], 6.0, 2e-5
+    cap, eps = 6.0, 2e-5
     T = sum(lengths)
     proj = rnd(g, T, 2 * H * d + 2 * H * dv).to(DT[dtype])
     gates = rnd(g, T, 2 * H, std=3.0).float()
@@ -103,8 +112,12 @@ def test_mlstm_carries_its_state_between_steps(dtype, H, d, dv):
     state[[2, 0, 3]] = 0.0
     got = torch.zeros((T, H * dv), dtype=torch.float64)
     for rows, cu, sl, _ in two_steps(lengths, cut):
+        pieces = None
+        if piece:
+            arr, n, multi = scan_pieces(cu, piece)
+            pieces = (i32(arr, dev), n, multi)
         y = ops.mlstm(proj[rows].to(dev), 0, H * d, 2 * H * d, 2 * H * d + H * dv, gates[rows].to(dev), bi.to(dev), bf.to(dev), cap,
-                      nw.to(dev), eps, state, i32(cu, dev), i32(sl, dev), H, d, dv)
+                      nw.to(dev), eps, state, i32(cu, dev), i32(sl, dev), H, d, dv, pieces=pieces)
         got[rows] = y.double().cpu()
     assert torch.isnan(state[1]).all()
     # the plain function with projections that hand the rows through: identity matrices behind a one-hot input
